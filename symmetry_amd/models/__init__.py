@@ -11,6 +11,10 @@ def model_class(cfg):
         from .lemunex import LemunexLM
 
         return LemunexLM
+    if family == "komazen":
+        from .komazen import KomazenLM
+
+        return KomazenLM
     if family == "llama":
         from .transformer import TransformerLM
 

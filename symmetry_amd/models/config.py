@@ -80,6 +80,9 @@ class LatentMixerSpec:
     rot_dims: int       # leading dims of the rotated part that turn (pairs 2i, 2i + 1)
     scale: float
     kv_from: int | None = None
+    window: int = 0             # > 0: a position sees itself and the window - 1 positions before it; 0: all before it
+    rot_half: bool = False      # rotary pairs dimension i with i + rot_dims / 2 instead of 2i with 2i + 1
+    gate: bool = False          # head outputs times sigmoid(W_g h), element by element
 
 
 @dataclass(frozen=True)
@@ -534,6 +537,195 @@ SMALL_LEMUNEX_MOE = lemunex_stack("small-lemunex-moe", 32768, 2048, "PMMP", head
                                   ff=8192, experts=16, top=4, identity=2, expert_ff=1024, shared_ff=2048,
                                   max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
 
+# --------------------------------------------------------------------------------------------------
+# Komazen: norm after the sum (x <- n(alpha x + sublayer(x))), a short causal convolution in front of every sublayer,
+# mixers: windowed latent attention (half-layout rotary, output gate, optional shared cache) or grouped-head softmax
+# attention with query / key norm, per-head temperature and a logarithmic distance bias; gelu-gated feed-forward.
+# --------------------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class BiasedAttnSpec:
+    """Causal softmax attention, no rotation: score = scale * temp_h * n(q) . n(k) - r1_h ln(1 + r2_h (i - j))."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+
+
+@dataclass(frozen=True)
+class GeluGluSpec:
+    ff: int
+
+
+@dataclass(frozen=True)
+class KomazenLayer:
+    type: str                    # "latent_attention" | "attention"
+    mixer: LatentMixerSpec | BiasedAttnSpec
+    mlp: GeluGluSpec | None = None
+
+
+@dataclass(frozen=True)
+class KomazenConfig:
+    family = "komazen"
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    embed_scale: float = 1.0
+    postln_alpha: float = 1.0
+    conv_taps: int = 4
+    norm_eps: float = 1e-5
+    max_position: int = 131072
+    bos_token_id: int = 1
+    eos_token_ids: tuple = (2,)
+    chat_format: str = "llama3"
+    tie_embeddings = False
+    rope_scaling = None
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return False
+
+    def latent_layers(self) -> list:
+        """Layers that own a plane of the paged latent cache (a down-projection of their own), in order."""
+        return [i for i, layer in enumerate(self.layers) if layer.type == "latent_attention" and layer.mixer.kv_from is None]
+
+    def attn_layers(self) -> list:
+        """Layers that own planes of the paged key / value cache, in order."""
+        return [i for i, layer in enumerate(self.layers) if layer.type == "attention"]
+
+    def num_params(self) -> int:
+        from .weights import komazen_shapes
+
+        n = 0
+        for shape in komazen_shapes(self).values():
+            k = 1
+            for v in shape:
+                k *= v
+            n += k
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        n = sum(self.layers[i].mixer.kv_rank + self.layers[i].mixer.rot_dim for i in self.latent_layers())
+        n += sum(self.layers[i].mixer.kv_heads * (self.layers[i].mixer.dim + self.layers[i].mixer.vdim)
+                 for i in self.attn_layers())
+        return n * dtype_bytes
+
+    def state_bytes_per_seq(self) -> int:
+        """The newest taps - 1 inputs of every sublayer's convolution (fp32)."""
+        subs = sum(1 + (layer.mlp is not None) for layer in self.layers)
+        return subs * (self.conv_taps - 1) * self.hidden_size * 4
+
+    def replace(self, **kw) -> "KomazenConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def komazen_from_config(cfg: dict, name: str = "komazen") -> KomazenConfig:
+    """config.json of a Komazen checkpoint: every size and constant is read here; a key this reader does not know means
+    a mechanism this code does not have, so it raises."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        kind, mixer, mlp = _take(L, f"layer {i}", "type", "mixer", optional=("mlp",))
+        if kind == "latent_attention":
+            dim, heads, r, mask, qr, rot, rd, scale, vdim, src = _take(
+                mixer, f"layer {i} mixer", "dim", "heads", "kv_rank", "mask", "q_rank", "rot", "rot_dim", "scale", "vdim",
+                optional=("kv_from",))
+            (window,) = _take(mask, f"layer {i} mask", "size")
+            base, dims = _take(rot, f"layer {i} rot", "base", "dims")
+            mix = LatentMixerSpec(heads=int(heads), dim=int(dim), rot_dim=int(rd), vdim=int(vdim), kv_rank=int(r),
+                                  q_rank=int(qr), rot_base=float(base), rot_dims=int(dims), scale=float(scale),
+                                  kv_from=None if src is None else int(src), window=int(window), rot_half=True, gate=True)
+            if mix.rot_dims > mix.rot_dim or mix.rot_dims % 2 or mix.rot_dim % 2 or mix.window < 1:
+                raise ValueError(f"layer {i}: rot.dims {dims} / rot_dim {rd} / mask.size {window} do not fit")
+            if mix.kv_from is not None:
+                s = layers[mix.kv_from] if 0 <= mix.kv_from < i else None
+                if s is None or s.type != "latent_attention" or s.mixer.kv_from is not None or (
+                        s.mixer.kv_rank, s.mixer.rot_dim, s.mixer.rot_base, s.mixer.rot_dims) != (
+                        mix.kv_rank, mix.rot_dim, mix.rot_base, mix.rot_dims):
+                    raise ValueError(f"layer {i}: kv_from {mix.kv_from} must name an earlier layer that owns a cache of "
+                                     "the same latent / rotary sizes")
+        elif kind == "attention":
+            dim, heads, kvh, scale, vdim = _take(mixer, f"layer {i} mixer", "dim", "heads", "kv_heads", "scale", "vdim")
+            mix = BiasedAttnSpec(int(heads), int(kvh), int(dim), int(vdim), float(scale))
+            if mix.heads % mix.kv_heads:
+                raise ValueError(f"layer {i}: heads {heads} / kv_heads {kvh} do not fit")
+        else:
+            raise ValueError(f"layer {i}: unknown layer type {kind!r}")
+        if mlp is None:
+            ff = None
+        elif mlp.get("kind") == "dense":
+            (_, f) = _take(mlp, f"layer {i} mlp", "kind", "ff")
+            ff = GeluGluSpec(int(f))
+        else:
+            raise ValueError(f"layer {i}: unknown mlp kind {mlp.get('kind')!r}")
+        layers.append(KomazenLayer(kind, mix, ff))
+    vocab, width, norm, _, canon, emb, alpha, _, bos, eos = _take(
+        cfg, "config", "vocab", "width", "norm", "layers", "canon", "embedding", "postln_alpha",
+        optional=("architecture", "bos_token_id", "eos_token_ids"))
+    (eps,) = _take(norm, "norm", "eps")
+    (taps,) = _take(canon, "canon", "taps")
+    (escale,) = _take(emb, "embedding", "scale")
+    if not 1 <= int(taps) <= 16:
+        raise ValueError(f"canon.taps {taps}: 1..16")
+    return KomazenConfig(name=name, vocab_size=int(vocab), hidden_size=int(width), layers=tuple(layers),
+                         embed_scale=float(escale), postln_alpha=float(alpha), conv_taps=int(taps), norm_eps=float(eps),
+                         bos_token_id=int(bos if bos is not None else 1),
+                         eos_token_ids=tuple(eos) if eos is not None else (2,))
+
+
+def komazen_to_config(c: KomazenConfig) -> dict:
+    """The config.json form of a KomazenConfig (exports, tests)."""
+    layers = []
+    for layer in c.layers:
+        m = layer.mixer
+        if layer.type == "latent_attention":
+            md = {"dim": m.dim, "heads": m.heads, "kv_rank": m.kv_rank, "mask": {"size": m.window}, "q_rank": m.q_rank,
+                  "rot": {"base": m.rot_base, "dims": m.rot_dims}, "rot_dim": m.rot_dim, "scale": m.scale, "vdim": m.vdim}
+            if m.kv_from is not None:
+                md["kv_from"] = m.kv_from
+        else:
+            md = {"dim": m.dim, "heads": m.heads, "kv_heads": m.kv_heads, "scale": m.scale, "vdim": m.vdim}
+        fd = None if layer.mlp is None else {"ff": layer.mlp.ff, "kind": "dense"}
+        layers.append({"mixer": md, "mlp": fd, "type": layer.type})
+    return {"architecture": "Komazen", "canon": {"taps": c.conv_taps}, "embedding": {"scale": c.embed_scale},
+            "layers": layers, "norm": {"eps": c.norm_eps}, "postln_alpha": c.postln_alpha, "vocab": c.vocab_size,
+            "width": c.hidden_size}
+
+
+def komazen_stack(name, vocab, width, pattern, heads, kv_heads, dim, ff, window=1024, rot_dim=64, kv_rank=512, q_rank=1536,
+                  vdim=None, embed_scale=1.0, postln_alpha=1.0, taps=4, **kw) -> KomazenConfig:
+    """A stack from a pattern string: "L" latent-attention layer with a cache of its own, "S" one that attends the
+    newest "L" layer's cache, "A" biased grouped-head attention; every layer with the gelu-gated feed-forward."""
+    layers, owner = [], None
+    vdim = vdim or dim
+    for i, ch in enumerate(pattern):
+        if ch in "LS":
+            if ch == "S" and owner is None:
+                raise ValueError("an S layer needs an L layer before it")
+            mix = LatentMixerSpec(heads, dim, rot_dim, vdim, kv_rank, q_rank, 10000.0, rot_dim, (dim + rot_dim) ** -0.5,
+                                  owner if ch == "S" else None, window, True, True)
+            if ch == "L":
+                owner = i
+            layers.append(KomazenLayer("latent_attention", mix, GeluGluSpec(ff)))
+        elif ch == "A":
+            layers.append(KomazenLayer("attention", BiasedAttnSpec(heads, kv_heads, dim, vdim, dim ** -0.5), GeluGluSpec(ff)))
+        else:
+            raise ValueError(f"pattern letter {ch!r}")
+    return KomazenConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), embed_scale=embed_scale,
+                         postln_alpha=postln_alpha, conv_taps=taps, **kw)
+
+
+TINY_KOMAZEN = komazen_stack("tiny-komazen", 512, 128, "LASA", heads=4, kv_heads=2, dim=16, ff=192, window=40, rot_dim=16,
+                             kv_rank=48, q_rank=40, vdim=24, embed_scale=8.0, postln_alpha=2.0, max_position=2048,
+                             bos_token_id=500, eos_token_ids=(501, 502))
+# layer shapes of a mid-size model (benchmarks; random weights)
+SMALL_KOMAZEN = komazen_stack("small-komazen", 32768, 2048, "LASA", heads=16, kv_heads=4, dim=128, ff=8192, window=1024,
+                              max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+
 LLAMA31_SCALING = {
     "rope_type": "llama3",
     "factor": 8.0,
@@ -576,7 +768,7 @@ _REGISTRY = {
     c.name: c
     for c in (LLAMA3_8B, LLAMA31_8B, LLAMA3_70B, LLAMA31_70B, MIXTRAL_8X7B, TINY_LLAMA, TINY_MIXTRAL, SMALL_LLAMA,
               TINY_LLAMA_KV8, TINY_MIXTRAL_E8, TINY_BOZEVIK, SMALL_BOZEVIK, SMALL_BOZEVIK_MOE, TINY_LEMUNEX,
-              SMALL_LEMUNEX, SMALL_LEMUNEX_MOE)
+              SMALL_LEMUNEX, SMALL_LEMUNEX_MOE, TINY_KOMAZEN, SMALL_KOMAZEN)
 }
 _ALIASES = {
     "llama3": "llama3:8b",
@@ -609,12 +801,14 @@ def known_models() -> list[str]:
 
 def from_config_json(cfg: dict, name: str = "hf", shapes: dict | None = None):
     """The model configuration of a checkpoint directory's config.json: the design is chosen by its
-    ``architecture`` key (Bozevik, Lemunex), otherwise the HuggingFace Llama / Mixtral keys.  ``shapes``: the
+    ``architecture`` key (Bozevik, Lemunex, Komazen), otherwise the HuggingFace Llama / Mixtral keys.  ``shapes``: the
     checkpoint's tensor shapes, for designs that leave some sizes to them."""
     if cfg.get("architecture") == "Bozevik":
         return bozevik_from_config(cfg, name)
     if cfg.get("architecture") == "Lemunex":
         return lemunex_from_config(cfg, name, shapes)
+    if cfg.get("architecture") == "Komazen":
+        return komazen_from_config(cfg, name)
     return from_hf_config(cfg, name)
 
 

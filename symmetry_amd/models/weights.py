@@ -182,6 +182,8 @@ def random_weights(cfg: ModelConfig, shard: ShardSpec | None = None, device="cpu
         return bozevik_random_weights(cfg, shard, device, dtype, seed)
     if getattr(cfg, "family", "llama") == "lemunex":
         return lemunex_random_weights(cfg, shard, device, dtype, seed)
+    if getattr(cfg, "family", "llama") == "komazen":
+        return komazen_random_weights(cfg, shard, device, dtype, seed)
     shard.validate(cfg)
     shapes = full_shapes(cfg)
     tensors = {}
@@ -238,6 +240,8 @@ def load_hf_weights(path: str, cfg: ModelConfig, shard: ShardSpec | None = None,
         return load_bozevik_weights(path, cfg, shard, device, dtype)
     if getattr(cfg, "family", "llama") == "lemunex":
         return load_lemunex_weights(path, cfg, shard, device, dtype)
+    if getattr(cfg, "family", "llama") == "komazen":
+        return load_komazen_weights(path, cfg, shard, device, dtype)
     shard.validate(cfg)
     wmap = _hf_index(path)
     handles = {}
@@ -533,5 +537,116 @@ def save_lemunex_checkpoint(weights: ModelWeights, path: str) -> None:
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(lemunex_to_config(weights.cfg), f, indent=1)
+    save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
+              os.path.join(path, "model.safetensors"))
+
+
+# --------------------------------------------------------------------------------------------------
+# Komazen checkpoints: tensors keep the checkpoint's names (embed, l<i>.norm1, l<i>.canon1, l<i>.mix.dq, l<i>.mix.q,
+# l<i>.mix.temp, l<i>.mlp.gate, ..., final.norm, head); models/komazen.py fuses what its GEMMs read.
+# --------------------------------------------------------------------------------------------------
+def komazen_shapes(cfg, optional: set | None = None) -> dict:
+    """Tensor name -> shape.  ``optional`` (a set) receives the names a checkpoint may carry without this code reading
+    them: the second norm and convolution of a layer that has no feed-forward."""
+    d = cfg.hidden_size
+    shapes = {"embed": (cfg.vocab_size, d), "final.norm": (d,), "head": (cfg.vocab_size, d)}
+    for i, layer in enumerate(cfg.layers):
+        p, m = f"l{i}.", layer.mixer
+        shapes[p + "norm1"] = (d,)
+        shapes[p + "canon1"] = (d, cfg.conv_taps)
+        if layer.type == "latent_attention":
+            shapes[p + "mix.dq"] = (m.q_rank, d)
+            shapes[p + "mix.dq.norm"] = (m.q_rank,)
+            shapes[p + "mix.uq"] = (m.heads * (m.dim + m.rot_dim), m.q_rank)
+            if m.kv_from is None:
+                shapes[p + "mix.dkv"] = (m.kv_rank + m.rot_dim, d)
+                shapes[p + "mix.dkv.norm"] = (m.kv_rank,)
+            shapes[p + "mix.uk"] = (m.heads * m.dim, m.kv_rank)
+            shapes[p + "mix.uv"] = (m.heads * m.vdim, m.kv_rank)
+            shapes[p + "mix.g"] = (m.heads * m.vdim, d)
+            shapes[p + "mix.o"] = (d, m.heads * m.vdim)
+        else:
+            shapes[p + "mix.q"] = (m.heads * m.dim, d)
+            shapes[p + "mix.k"] = (m.kv_heads * m.dim, d)
+            shapes[p + "mix.v"] = (m.kv_heads * m.vdim, d)
+            shapes[p + "mix.q.norm"] = (m.dim,)
+            shapes[p + "mix.k.norm"] = (m.dim,)
+            for nm in ("r1", "r2", "temp"):
+                shapes[p + "mix." + nm] = (m.heads,)
+            shapes[p + "mix.o"] = (d, m.heads * m.vdim)
+        if layer.mlp is not None:
+            f = layer.mlp.ff
+            shapes[p + "norm2"] = (d,)
+            shapes[p + "canon2"] = (d, cfg.conv_taps)
+            shapes[p + "mlp.gate"], shapes[p + "mlp.up"], shapes[p + "mlp.down"] = (f, d), (f, d), (d, f)
+        elif optional is not None:
+            optional.update((p + "norm2", p + "canon2"))
+    return shapes
+
+
+def komazen_random_weights(cfg, shard: ShardSpec | None = None, device="cpu", dtype=torch.bfloat16,
+                           seed: int = 0) -> ModelWeights:
+    """Random init (benchmarks, tests): matrices N(0, (1.28 / sqrt(fan_in))^2); norm weights around one; convolution
+    taps small and of both signs; temperatures around one, distance-bias parameters positive -- all away from the
+    values at which a dropped parameter would not show (1 for a factor, 0 for a term)."""
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Komazen runs on one GPU per replica (its tensors are not sharded)")
+    tensors = {}
+    for name, shape in komazen_shapes(cfg).items():
+        g = torch.Generator().manual_seed(_seed(seed, name))
+        if "canon" in name:
+            t = (torch.rand(shape, generator=g) - 0.5) * 0.6
+        elif name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
+            t = 0.75 + 0.5 * torch.rand(shape, generator=g)
+        elif name.endswith(".temp"):
+            t = 0.6 + 0.8 * torch.rand(shape, generator=g)
+        elif name.endswith(".r1"):
+            t = 0.2 + 0.8 * torch.rand(shape, generator=g)
+        elif name.endswith(".r2"):
+            t = 0.05 + 0.5 * torch.rand(shape, generator=g)
+        else:
+            t = None
+        if t is not None:
+            tensors[name] = t.to(dtype).to(device)
+        else:
+            tensors[name] = _randn(shape, _seed(seed, name), device, dtype, 1.0 if name == "embed" else _std(name, shape))
+    return ModelWeights(cfg, shard, tensors)
+
+
+def load_komazen_weights(path: str, cfg, shard: ShardSpec | None = None, device="cpu",
+                         dtype=torch.bfloat16) -> ModelWeights:
+    """model.safetensors of a Komazen checkpoint directory; every tensor the configuration implies must be there with
+    the implied shape, and no other.  Tensors stay in the file's precision (the model converts what it fuses)."""
+    from safetensors import safe_open
+
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Komazen runs on one GPU per replica (its tensors are not sharded)")
+    optional: set = set()
+    shapes = komazen_shapes(cfg, optional)
+    tensors = {}
+    with safe_open(os.path.join(path, "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+        missing, extra = sorted(set(shapes) - names), sorted(names - set(shapes) - optional)
+        if missing or extra:
+            raise ValueError(f"checkpoint does not fit its config: missing {missing[:4]}, unexpected {extra[:4]}")
+        for name, shape in shapes.items():
+            t = f.get_tensor(name)
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"{name}: shape {tuple(t.shape)}, the config implies {tuple(shape)}")
+            tensors[name] = t.to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def save_komazen_checkpoint(weights: ModelWeights, path: str) -> None:
+    """config.json + model.safetensors (bf16) of a Komazen model, in the form the loader reads."""
+    from safetensors.torch import save_file
+
+    from .config import komazen_to_config
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(komazen_to_config(weights.cfg), f, indent=1)
     save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
               os.path.join(path, "model.safetensors"))

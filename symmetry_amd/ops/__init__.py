@@ -624,20 +624,23 @@ def rope_pair_table(max_pos: int, dims: int, base: float, device=None) -> torch.
     return reference.rope_pair_table(max_pos, dims, base, device)
 
 
-def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache):
-    """z [T, q_rank (+ kv_rank + rot)] -> cq = rms_norm(z[:, :q_rank]) * wq; with a kv part (kv_rank > 0) the token's
-    cache row (slot >= 0) becomes [rms_norm(z kv part) * wkv | rotary(z rot part)]."""
+def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache, half_dims=0):
+    """z [T, q_rank (+ kv_rank + rot)] (a view: further columns may follow in its rows) -> cq = rms_norm(z[:, :q_rank]) *
+    wq; with a kv part (kv_rank > 0) the token's cache row (slot >= 0) becomes [rms_norm(z kv part) * wkv | rotary(z rot
+    part)].  ``half_dims`` = 0: rotary pairs (2i, 2i + 1); > 0: the half layout, entry i < half_dims / 2 paired with
+    i + half_dims / 2 and the entries past half_dims passing."""
     if _gpu(z):
         return _lat().latent_prep(z, int(q_rank), int(kv_rank), int(rot), wq, wkv, float(eps), positions, slots, rope,
-                                  cq, cache)
-    return reference.latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache)
+                                  cq, cache, int(half_dims))
+    return reference.latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache, half_dims)
 
 
-def rope_pairs(src, dst, positions, rope):
-    """Interleaved-pair rotary of a [T, H, rot] view into another (unit inner strides)."""
+def rope_pairs(src, dst, positions, rope, half_dims=0):
+    """Rotary of a [T, H, rot] view into another (unit inner strides): interleaved pairs, or with ``half_dims`` > 0 the
+    half layout (entry i with i + half_dims / 2)."""
     if _gpu(src):
-        return _lat().rope_pairs(src, dst, positions, rope)
-    return reference.rope_pairs(src, dst, positions, rope)
+        return _lat().rope_pairs(src, dst, positions, rope, int(half_dims))
+    return reference.rope_pairs(src, dst, positions, rope, half_dims)
 
 
 def latent_attn_parts(rows: int, span: int, target_wgs: int = 512, min_tokens: int = 64) -> int:
@@ -650,7 +653,7 @@ LATENT_ATTN_IMPL = 1 if os.environ.get("SYMMETRY_LATENT_ATTN", "mfma") == "wave"
 
 
 def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, part_o=None, part_ml=None,
-                tiles=None, cu_q=None, impl=None):
+                tiles=None, cu_q=None, impl=None, window=0):
     """Causal softmax attention of q [T, H, Dk] over the paged latent cache [NB, BS, Dk]: keys are whole cache rows,
     values their first kv_rank entries; row r sees keys 0..positions[r] of sequence row_seq[r].  ``part_o``
     [T, H, parts, kv_rank] / ``part_ml`` [T, H, parts, 2]: split-KV scratch (decode steps: ``parts`` equal partitions of
@@ -658,11 +661,13 @@ def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out,
     ``tiles`` [n, 2] (sequence, first row of a 64-row tile within the sequence's run) + ``cu_q``: the prompt form of
     the MFMA kernel (bf16, Dk % 32 == 0, kv_rank % 16 == 0); without them that kernel takes one row per sequence
     (decode steps).  Other shapes, fp32 and ``impl=1`` run the one-wave-per-(row, head) kernel.  Returns the
-    implementation used (0 MFMA, 1 wave)."""
+    implementation used (0 MFMA, 1 wave).  ``window`` > 0: row r sees only the keys positions[r] - window + 1 ..
+    positions[r], and the split-KV partitions cover that range (count them with ``latent_attn_parts(rows, min(span,
+    window))``)."""
     if _gpu(q):
         return _lat().latent_attn(q, cache, block_tables, row_seq, positions, float(scale), int(kv_rank), out, part_o,
-                                  part_ml, tiles, cu_q, LATENT_ATTN_IMPL if impl is None else int(impl))
-    reference.latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out)
+                                  part_ml, tiles, cu_q, LATENT_ATTN_IMPL if impl is None else int(impl), int(window))
+    reference.latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, window)
     return 1
 
 
@@ -759,16 +764,17 @@ WINDOW_ATTN_IMPL = 0 if os.environ.get("SYMMETRY_WINDOW_ATTN", "auto") == "wave"
 
 
 def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, tiles=None, cu_q=None,
-                impl=None):
+                impl=None, bias=None):
     """Softmax attention of q [T, H, dk] over the paged caches: row r sees positions max(0, p - window + 1) .. p of
     sequence row_seq[r] (p = positions[r]); query head h reads key / value head h // (H / G); scores and weights
     fp32.  ``gate`` [T, H] (a view): head outputs are multiplied by sigmoid(gate).  ``tiles`` / ``cu_q``: the packed
     prompt form (64-row query tiles), for the tiled kernel.  Returns the implementation used (0: one wave per (row,
-    head), every shape; 1: tiled)."""
+    head), every shape; 1: tiled).  ``bias`` [2, H] fp32: the score of a key at distance n = p - j is lowered by
+    bias[0, h] * ln(1 + bias[1, h] * n)."""
     if _gpu(q):
         return _hyb().window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, int(window), float(scale), gate,
-                                  out, tiles, cu_q, WINDOW_ATTN_IMPL if impl is None else int(impl))
-    reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out)
+                                  out, tiles, cu_q, WINDOW_ATTN_IMPL if impl is None else int(impl), bias)
+    reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias)
     return 0
 
 
@@ -859,3 +865,51 @@ def hyb_grouped_linear(xs, W, offsets, y):
     if _gpu(xs):
         return _hyb().grouped_linear(xs, W, offsets, y)
     return reference.grouped_linear(xs, W, offsets, y)
+
+
+# ---- post-norm stream, input convolutions, normed grouped heads (csrc/kernels/hybrid_rows.hip) ---------------------
+def embed_scale(ids, table, scale, x, src=None, prev=None):
+    """x (fp32) = table[token] * scale; rows with src >= 0 take the token prev[src]."""
+    if _gpu(x):
+        return _hyb().embed_scale(ids, src, prev, table, float(scale), x)
+    return reference.embed_scale(reference.resolve_ids(ids, src, prev), table, scale, x)
+
+
+def residual_conv(x, w, state, cu_q, row_seq, prev_row, runs, out):
+    """out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j) per channel over every run of rows of the fp32 stream x (the
+    sublayer input in the activation dtype); inputs before the run come from state[slot] [taps - 1, C] fp32
+    (prev_row[first] <= -2) or are zero.  ``conv_state_update(x, state, ...)`` then stores the run's newest inputs."""
+    if _gpu(out):
+        return _hyb().residual_conv(x, w, state, cu_q, row_seq if cu_q is not None else None, prev_row, int(runs), out)
+    return reference.residual_conv(x, w, state, cu_q, prev_row, runs, out)
+
+
+def post_rms_norm(x, alpha, delta, w, eps):
+    """Norm after the sum, in place on the fp32 stream: x = (alpha x + delta) / rms(alpha x + delta) * w."""
+    if _gpu(x):
+        return _hyb().post_rms_norm(x, float(alpha), delta, w, float(eps))
+    return reference.post_rms_norm(x, alpha, delta, w, eps)
+
+
+def qk_norm_cache(z, H, G, dk, dv, wq, wk, q_mult, eps, slots, q_out, k_cache, v_cache):
+    """z [T, H dk | G dk | G dv (| ...)] -> q_out [T, H, dk] = rms_norm per head (weight wq [dk], shared by the heads)
+    times q_mult[h] (optional); the token's rows of the paged caches k [NB, BS, G, dk] = rms_norm per head (wk),
+    v [NB, BS, G, dv] (slot >= 0).  Statistics fp32."""
+    if _gpu(z):
+        return _hyb().qk_norm_cache(z, int(H), int(G), int(dk), int(dv), wq, wk, q_mult, float(eps), slots, q_out,
+                                    k_cache, v_cache)
+    return reference.qk_norm_cache(z, H, G, dk, dv, wq, wk, q_mult, eps, slots, q_out, k_cache, v_cache)
+
+
+def gelu_tanh_mul(gate, up, out):
+    """out = gelu(gate) * up with the tanh form 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))); [R, F] views."""
+    if _gpu(out):
+        return _hyb().gelu_tanh_mul(gate, up, out)
+    return reference.gelu_tanh_mul(gate, up, out)
+
+
+def sigmoid_mul(a, gate, out):
+    """out = a * sigmoid(gate), element by element ([R, F]; gate a view; out may be a)."""
+    if _gpu(out):
+        return _hyb().sigmoid_mul(a, gate, out)
+    return reference.sigmoid_mul(a, gate, out)

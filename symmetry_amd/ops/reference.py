@@ -618,7 +618,19 @@ def _rot_pairs(v, cs):
     return torch.stack([u * c - w * s, w * c + u * s], -1).flatten(-2)
 
 
-def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache) -> None:
+def _rot_half(v, cs, dims):
+    """Half layout: entry i < dims / 2 pairs with entry i + dims / 2 (table pair i); entries past ``dims`` pass."""
+    h = dims // 2
+    u, w = v[..., :h], v[..., h:dims]
+    c, s = cs[..., :h, 0], cs[..., :h, 1]
+    return torch.cat([u * c - w * s, w * c + u * s, v[..., dims:]], -1)
+
+
+def _rot(v, cs, half_dims):
+    return _rot_half(v, cs, half_dims) if half_dims else _rot_pairs(v, cs)
+
+
+def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache, half_dims=0) -> None:
     T = z.shape[0]
     zf = z.float()
     q = zf[:, :q_rank]
@@ -627,26 +639,26 @@ def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, c
         return
     c = zf[:, q_rank:q_rank + kv_rank]
     c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * wkv.float()
-    kr = _rot_pairs(zf[:, q_rank + kv_rank:], rope[positions[:T].long()])
+    kr = _rot(zf[:, q_rank + kv_rank:q_rank + kv_rank + rot], rope[positions[:T].long()], half_dims)
     row = torch.cat([c, kr], -1).to(cache.dtype)
     sl = slots[:T].long()
     keep = sl >= 0
     cache.view(-1, kv_rank + rot)[sl[keep]] = row[keep]
 
 
-def rope_pairs(src, dst, positions, rope) -> None:
+def rope_pairs(src, dst, positions, rope, half_dims=0) -> None:
     T = src.shape[0]
-    dst.copy_(_rot_pairs(src.float(), rope[positions[:T].long()][:, None]).to(dst.dtype))
+    dst.copy_(_rot(src.float(), rope[positions[:T].long()][:, None], half_dims).to(dst.dtype))
 
 
-def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out) -> None:
+def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, window=0) -> None:
     T, H, Dk = q.shape
     BS = cache.shape[1]
     o = out.view(T, H, kv_rank)
     for r in range(T):
         n = int(positions[r]) + 1
         bt = block_tables[int(row_seq[r])].long()
-        idx = torch.arange(n)
+        idx = torch.arange(max(0, n - window) if window > 0 else 0, n)
         rows = cache[bt[idx // BS], idx % BS].float()          # [n, Dk]
         s = (q[r].float() @ rows.t()) * scale                   # [H, n]
         p = torch.softmax(s, -1)
@@ -775,7 +787,7 @@ def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache
     v_cache.view(-1, G, dv)[sl[keep]] = v[keep]
 
 
-def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out) -> None:
+def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias=None) -> None:
     T, H, dk = q.shape
     BS, G = k_cache.shape[1], k_cache.shape[2]
     rep = H // G
@@ -788,6 +800,9 @@ def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, s
         V = v_cache[bt[idx // BS], idx % BS].float()
         qr = q[r].float().view(G, rep, dk)
         s = torch.einsum("grd,ngd->grn", qr, K) * scale
+        if bias is not None:     # [2, H]: score -= bias[0, h] * ln(1 + bias[1, h] * distance)
+            dist = (p - idx).float()
+            s = s - (bias[0].float()[:, None] * torch.log1p(bias[1].float()[:, None] * dist[None, :])).view(G, rep, -1)
         o = torch.einsum("grn,ngv->grv", torch.softmax(s, -1), V).reshape(H, -1)
         if gate is not None:
             o = o * torch.sigmoid(gate[r].float())[:, None]
@@ -900,3 +915,54 @@ def moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out) -> None:
     if shared is not None:
         s = s + torch.sigmoid(sgate.float()).view(T, 1) * shared.float().view_as(s)
     out.copy_(s)
+
+
+# ---- post-norm stream, input convolutions, normed grouped heads (the Komazen layers) ----------------------------
+def embed_scale(ids, table, scale, x) -> None:
+    x.copy_(table[ids.long()].float() * scale)
+
+
+def residual_conv(x, w, state, cu_q, prev_row, runs, out) -> None:
+    T, C = out.shape
+    taps = w.shape[1]
+    wf = w.float()
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 <= s0:
+            continue
+        pr = int(prev_row[s0])
+        hist = state[-(pr + 2)].float() if pr <= -2 else torch.zeros(taps - 1, C)
+        full = torch.cat([hist, x[s0:s1]], 0)
+        y = x[s0:s1].clone()
+        for j in range(taps):
+            y = y + full[j:j + s1 - s0] * wf[:, j]
+        out[s0:s1] = y.to(out.dtype)
+
+
+def post_rms_norm(x, alpha, delta, w, eps) -> None:
+    x.copy_(_unit_rms(alpha * x + delta.float().view_as(x), eps) * w.float())
+
+
+def qk_norm_cache(z, H, G, dk, dv, wq, wk, q_mult, eps, slots, q_out, k_cache, v_cache) -> None:
+    T = z.shape[0]
+    nq, nk, nv = H * dk, G * dk, G * dv
+    zf = z[:, :nq + nk + nv].float()
+    q = _unit_rms(zf[:, :nq].view(T, H, dk), eps) * wq.float()
+    if q_mult is not None:
+        q = q * q_mult.float()[None, :, None]
+    q_out.copy_(q.to(q_out.dtype))
+    k = (_unit_rms(zf[:, nq:nq + nk].view(T, G, dk), eps) * wk.float()).to(k_cache.dtype)
+    v = zf[:, nq + nk:].view(T, G, dv).to(v_cache.dtype)
+    sl = slots[:T].long()
+    keep = sl >= 0
+    k_cache.view(-1, G, dk)[sl[keep]] = k[keep]
+    v_cache.view(-1, G, dv)[sl[keep]] = v[keep]
+
+
+def gelu_tanh_mul(gate, up, out) -> None:
+    g = gate.float()
+    act = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g)))
+    out.copy_((act * up.float()).to(out.dtype))
+
+
+def sigmoid_mul(a, gate, out) -> None:
+    out.copy_((a.float() * torch.sigmoid(gate.float())).to(out.dtype))
