@@ -175,7 +175,7 @@ void qkv_rope_cache(const Tensor& z, const Tensor& bias, int64_t H, int64_t G, i
 
 int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_tables,
                     const Tensor& row_seq, const Tensor& positions, int64_t window, double scale, const OptTensor& gate,
-                    Tensor& out, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl) {
+                    Tensor& out, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl, const OptTensor& bias) {
   const int f32 = act(q, "q");
   same_act(k_cache, f32, "k_cache");
   same_act(v_cache, f32, "v_cache");
@@ -196,6 +196,11 @@ int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cach
   if (gate.has_value()) {
     a.ldg = view2(*gate, f32, a.T, a.H, "gate");
     a.gate = gate->data_ptr();
+  }
+  if (bias.has_value()) {
+    dtype(*bias, at::kFloat, "bias");
+    TORCH_CHECK(bias->dim() == 2 && bias->size(0) == 2 && bias->size(1) == a.H, "window_attn: bias [2, H]");
+    a.bias = ptr<float>(*bias);
   }
   if (tiles.has_value() && cu_q.has_value()) {
     dtype(*tiles, at::kInt, "tiles");
@@ -443,6 +448,99 @@ void grouped_linear(const Tensor& xs, const Tensor& W, const Tensor& offsets, Te
                         cur_stream(xs));
 }
 
+// ---- post-norm stream, input convolutions, normed grouped heads ---------------------------------------------------
+void embed_scale(const Tensor& ids, const OptTensor& src, const OptTensor& prev, const Tensor& table, double scale,
+                 Tensor& x) {
+  const int f32 = act(table, "table");
+  dtype(ids, at::kInt, "ids");
+  dtype(x, at::kFloat, "x");
+  const int64_t T = ids.numel(), d = table.size(1);
+  TORCH_CHECK(table.dim() == 2 && x.numel() == T * d, "embed_scale: shapes");
+  if (src.has_value()) {
+    TORCH_CHECK(prev.has_value(), "embed_scale: src without prev");
+    dtype(*src, at::kInt, "src");
+    dtype(*prev, at::kInt, "prev");
+    TORCH_CHECK(src->numel() >= T, "embed_scale: src too short");
+  }
+  launch_embed_scale(ptr<int>(ids), optptr<int>(src), optptr<int>(prev), table.data_ptr(), (float)scale, ptr<float>(x),
+                     (int)T, (int)d, f32, cur_stream(x));
+}
+
+void residual_conv(const Tensor& x, const Tensor& w, Tensor& state, const OptTensor& cu_q, const OptTensor& row_seq,
+                   const Tensor& prev_row, int64_t runs, Tensor& out) {
+  const int f32 = act(out, "out");
+  dtype(x, at::kFloat, "x");
+  dtype(w, at::kFloat, "w");
+  dtype(state, at::kFloat, "state");
+  ConvArgs a = conv_args(x, w, std::nullopt, state, cu_q, row_seq, prev_row, std::nullopt, runs, 1);
+  TORCH_CHECK(!cu_q.has_value() || row_seq.has_value(), "residual_conv: cu_q without row_seq");
+  TORCH_CHECK(out.numel() == (int64_t)a.T * a.C, "residual_conv: out shape");
+  a.out = out.data_ptr();
+  launch_residual_conv(a, f32, cur_stream(out));
+}
+
+void post_rms_norm(Tensor& x, double alpha, const Tensor& delta, const Tensor& w, double eps) {
+  const int f32 = act(delta, "delta");
+  dtype(x, at::kFloat, "x");
+  dtype(w, at::kFloat, "w");
+  TORCH_CHECK(x.dim() == 2 && delta.numel() == x.numel() && w.numel() == x.size(1), "post_rms_norm: x [T, d], delta [T, d]");
+  launch_post_rms_norm(ptr<float>(x), (float)alpha, delta.data_ptr(), ptr<float>(w), (float)eps, (int)x.size(0),
+                       (int)x.size(1), f32, cur_stream(x));
+}
+
+void qk_norm_cache(const Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const Tensor& wq, const Tensor& wk,
+                   const OptTensor& q_mult, double eps, const Tensor& slots, Tensor& q_out, Tensor& k_cache,
+                   Tensor& v_cache) {
+  const int f32 = act(z, "z", false);
+  TORCH_CHECK(z.dim() == 2, "qk_norm_cache: z [T, n]");
+  const int64_t T = z.size(0), n = H * dk + G * dk + G * dv;
+  QkNormArgs a{};
+  a.ldz = view2(z, f32, T, z.size(1), "z");
+  TORCH_CHECK(z.size(1) >= n, "qk_norm_cache: z narrower than q | k | v");
+  same_act(q_out, f32, "q_out");
+  same_act(k_cache, f32, "k_cache");
+  same_act(v_cache, f32, "v_cache");
+  dtype(wq, at::kFloat, "wq");
+  dtype(wk, at::kFloat, "wk");
+  dtype(slots, at::kInt, "slots");
+  TORCH_CHECK(wq.numel() == dk && wk.numel() == dk && q_out.numel() == T * H * dk && slots.numel() >= T &&
+                  k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(2) == G && k_cache.size(3) == dk &&
+                  v_cache.size(2) == G && v_cache.size(3) == dv && G > 0 && H % G == 0 && T <= 65535 * 64 && H + G <= 65535,
+              "qk_norm_cache: shapes");
+  if (q_mult.has_value()) {
+    dtype(*q_mult, at::kFloat, "q_mult");
+    TORCH_CHECK(q_mult->numel() == H, "qk_norm_cache: q_mult [H]");
+    a.q_mult = ptr<float>(*q_mult);
+  }
+  a.z = z.data_ptr();
+  a.H = (int)H, a.G = (int)G, a.dk = (int)dk, a.dv = (int)dv;
+  a.wq = ptr<float>(wq), a.wk = ptr<float>(wk);
+  a.eps = (float)eps;
+  a.slots = ptr<int>(slots);
+  a.q_out = q_out.data_ptr();
+  a.k_cache = k_cache.data_ptr();
+  a.v_cache = v_cache.data_ptr();
+  launch_qk_norm_cache(a, (int)T, f32, cur_stream(z));
+}
+
+void gelu_tanh_mul(const Tensor& gate, const Tensor& up, Tensor& out) {
+  const int f32 = act(out, "out");
+  TORCH_CHECK(out.dim() == 2, "gelu_tanh_mul: out [R, F]");
+  const int64_t ldg = view2(gate, f32, out.size(0), out.size(1), "gate");
+  const int64_t ldu = view2(up, f32, out.size(0), out.size(1), "up");
+  launch_gelu_tanh_mul(gate.data_ptr(), ldg, up.data_ptr(), ldu, out.data_ptr(), (int)out.size(0), (int)out.size(1), f32,
+                       cur_stream(out));
+}
+
+void sigmoid_mul(const Tensor& a, const Tensor& gate, Tensor& out) {
+  const int f32 = act(out, "out");
+  TORCH_CHECK(out.dim() == 2, "sigmoid_mul: out [R, F]");
+  const int64_t lda = view2(a, f32, out.size(0), out.size(1), "a");
+  const int64_t ldg = view2(gate, f32, out.size(0), out.size(1), "gate");
+  launch_sigmoid_mul(a.data_ptr(), lda, gate.data_ptr(), ldg, out.data_ptr(), (int)out.size(0), (int)out.size(1), f32,
+                     cur_stream(out));
+}
+
 }  // namespace
 
 TORCH_LIBRARY(symmetry_amd_hybrid, m) {
@@ -459,7 +557,7 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
       &qkv_rope_cache);
   m.def(
       "window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor row_seq, Tensor positions, "
-      "int window, float scale, Tensor? gate, Tensor(a!) out, Tensor? tiles, Tensor? cu_q, int impl) -> int",
+      "int window, float scale, Tensor? gate, Tensor(a!) out, Tensor? tiles, Tensor? cu_q, int impl, Tensor? bias) -> int",
       &window_attn);
   m.def(
       "decay_scan(int mode, Tensor q, Tensor k, Tensor v, Tensor dz, Tensor dbias, Tensor? rate, float tau, Tensor? skip, "
@@ -487,4 +585,16 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
       "Tensor(c!) dst) -> ()",
       &scatter_scaled);
   m.def("grouped_linear(Tensor xs, Tensor W, Tensor offsets, Tensor(a!) y) -> ()", &grouped_linear);
+  m.def("embed_scale(Tensor ids, Tensor? src, Tensor? prev, Tensor table, float scale, Tensor(a!) x) -> ()", &embed_scale);
+  m.def(
+      "residual_conv(Tensor x, Tensor w, Tensor(a!) state, Tensor? cu_q, Tensor? row_seq, Tensor prev_row, int runs, "
+      "Tensor(b!) out) -> ()",
+      &residual_conv);
+  m.def("post_rms_norm(Tensor(a!) x, float alpha, Tensor delta, Tensor w, float eps) -> ()", &post_rms_norm);
+  m.def(
+      "qk_norm_cache(Tensor z, int H, int G, int dk, int dv, Tensor wq, Tensor wk, Tensor? q_mult, float eps, Tensor slots, "
+      "Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()",
+      &qk_norm_cache);
+  m.def("gelu_tanh_mul(Tensor gate, Tensor up, Tensor(a!) out) -> ()", &gelu_tanh_mul);
+  m.def("sigmoid_mul(Tensor a, Tensor gate, Tensor(a!) out) -> ()", &sigmoid_mul);
 }

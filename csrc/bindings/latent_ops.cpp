@@ -135,8 +135,8 @@ void layer_norm(const Tensor& x, const OptTensor& rows, const Tensor& w, double 
 
 void latent_prep(const Tensor& z, int64_t q_rank, int64_t kv_rank, int64_t rot, const Tensor& wq, const OptTensor& wkv,
                  double eps, const Tensor& positions, const Tensor& slots, const Tensor& rope, Tensor& cq,
-                 const OptTensor& cache) {
-  const int f32 = act(z, "z");
+                 const OptTensor& cache, int64_t half_dims) {
+  const int f32 = act(z, "z", false);
   same_act(wq, f32, "wq");
   same_act(cq, f32, "cq");
   dtype(positions, at::kInt, "positions");
@@ -145,7 +145,11 @@ void latent_prep(const Tensor& z, int64_t q_rank, int64_t kv_rank, int64_t rot, 
   const int64_t T = z.size(0);
   LatentPrepArgs a{};
   a.z = z.data_ptr();
-  a.nz = (int)z.size(1);
+  TORCH_CHECK(z.dim() == 2 && (z.size(1) == 1 || z.stride(1) == 1), "latent_prep: z [T, n] with unit inner stride");
+  a.nz = (int)(T > 1 ? z.stride(0) : z.size(1));
+  const int64_t zcols = z.size(1);
+  TORCH_CHECK(half_dims >= 0 && half_dims % 2 == 0 && half_dims <= rot, "latent_prep: half_dims");
+  a.half_dims = (int)half_dims;
   a.q_rank = (int)q_rank;
   a.kv_rank = (int)kv_rank;
   a.rot = (int)rot;
@@ -155,12 +159,12 @@ void latent_prep(const Tensor& z, int64_t q_rank, int64_t kv_rank, int64_t rot, 
     TORCH_CHECK(wkv.has_value() && cache.has_value(), "latent_prep: kv part needs wkv and cache");
     same_act(*wkv, f32, "wkv");
     same_act(*cache, f32, "cache");
-    TORCH_CHECK(a.nz == q_rank + kv_rank + rot && wkv->numel() == kv_rank && cache->size(-1) == kv_rank + rot &&
+    TORCH_CHECK(zcols == q_rank + kv_rank + rot && wkv->numel() == kv_rank && cache->size(-1) == kv_rank + rot &&
                     rope.dim() == 3 && rope.size(1) == rot / 2 && rope.size(2) == 2, "latent_prep: kv shapes");
     a.wkv = wkv->data_ptr();
     a.cache = cache->data_ptr();
   } else {
-    TORCH_CHECK(a.nz == q_rank, "latent_prep: z width");
+    TORCH_CHECK(zcols == q_rank, "latent_prep: z width");
   }
   a.wq = wq.data_ptr();
   a.eps = (float)eps;
@@ -171,7 +175,7 @@ void latent_prep(const Tensor& z, int64_t q_rank, int64_t kv_rank, int64_t rot, 
   launch_latent_prep(a, (int)T, f32, cur_stream(z));
 }
 
-void rope_pairs(const Tensor& src, Tensor& dst, const Tensor& positions, const Tensor& rope) {
+void rope_pairs(const Tensor& src, Tensor& dst, const Tensor& positions, const Tensor& rope, int64_t half_dims) {
   const int f32 = act(src, "src", false);
   same_act(dst, f32, "dst", false);
   dtype(positions, at::kInt, "positions");
@@ -179,15 +183,15 @@ void rope_pairs(const Tensor& src, Tensor& dst, const Tensor& positions, const T
   TORCH_CHECK(src.dim() == 3 && dst.dim() == 3 && src.sizes() == dst.sizes() && src.stride(2) == 1 && dst.stride(2) == 1,
               "rope_pairs: [T, H, rot] views with unit inner stride");
   const int64_t T = src.size(0), H = src.size(1), rot = src.size(2);
-  TORCH_CHECK(rot % 2 == 0 && rope.dim() == 3 && rope.size(1) == rot / 2 && rope.size(2) == 2 && positions.numel() >= T,
-              "rope_pairs: table / positions");
+  TORCH_CHECK(rot % 2 == 0 && rope.dim() == 3 && rope.size(1) == rot / 2 && rope.size(2) == 2 && positions.numel() >= T &&
+                  half_dims >= 0 && half_dims % 2 == 0 && half_dims <= rot, "rope_pairs: table / positions / half_dims");
   launch_rope_pairs(src.data_ptr(), src.stride(0), src.stride(1), dst.data_ptr(), dst.stride(0), dst.stride(1),
-                    ptr<int>(positions), ptr<float>(rope), (int)T, (int)H, (int)rot, f32, cur_stream(src));
+                    ptr<int>(positions), ptr<float>(rope), (int)T, (int)H, (int)rot, (int)half_dims, f32, cur_stream(src));
 }
 
 int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_tables, const Tensor& row_seq,
                     const Tensor& positions, double scale, int64_t kv_rank, Tensor& out, const OptTensor& part_o,
-                    const OptTensor& part_ml, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl) {
+                    const OptTensor& part_ml, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl, int64_t window) {
   const int f32 = act(q, "q");
   same_act(cache, f32, "cache");
   same_act(out, f32, "out");
@@ -207,7 +211,8 @@ int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_ta
     if ((1 << sh) == a.BS) a.bs_shift = sh;
   TORCH_CHECK(cache.size(2) == a.Dk && kv_rank > 0 && kv_rank <= a.Dk && kv_rank <= 512 && a.Dk <= 8192 &&
                   out.numel() == (int64_t)a.T * a.H * kv_rank && row_seq.numel() >= a.T && positions.numel() >= a.T &&
-                  a.H <= 65535, "latent_attn: shapes");
+                  a.H <= 65535 && window >= 0, "latent_attn: shapes");
+  a.window = (int)std::min<int64_t>(window, 1 << 30);
   a.parts = 1;
   a.part_tokens = 32;
   if (part_o.has_value()) {
@@ -218,7 +223,8 @@ int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_ta
     TORCH_CHECK(part_o->dim() == 4 && part_o->size(0) == a.T && part_o->size(1) == a.H && part_o->size(3) == kv_rank &&
                     part_ml->numel() == (int64_t)a.T * a.H * part_o->size(2) * 2, "latent_attn: partial buffer shapes");
     a.parts = (int)part_o->size(2);
-    const int64_t span = (int64_t)a.max_blocks * a.BS;
+    // (with a window a row's partitions start at its first visible key and cover at most the window)
+    const int64_t span = a.window > 0 ? std::min<int64_t>((int64_t)a.max_blocks * a.BS, a.window) : (int64_t)a.max_blocks * a.BS;
     a.part_tokens = (int)(((span + a.parts - 1) / a.parts + 31) / 32 * 32);
     TORCH_CHECK(a.parts >= 1 && a.parts <= 1024 && (int64_t)a.parts * a.part_tokens >= span, "latent_attn: partitions");
     a.part_o = ptr<float>(*part_o);
@@ -332,12 +338,13 @@ TORCH_LIBRARY(symmetry_amd_latent, m) {
   m.def("layer_norm(Tensor x, Tensor? rows, Tensor w, float eps, Tensor(a!) out) -> ()", &layer_norm);
   m.def(
       "latent_prep(Tensor z, int q_rank, int kv_rank, int rot, Tensor wq, Tensor? wkv, float eps, Tensor positions, "
-      "Tensor slots, Tensor rope, Tensor(a!) cq, Tensor(b!)? cache) -> ()",
+      "Tensor slots, Tensor rope, Tensor(a!) cq, Tensor(b!)? cache, int half_dims) -> ()",
       &latent_prep);
-  m.def("rope_pairs(Tensor src, Tensor(a!) dst, Tensor positions, Tensor rope) -> ()", &rope_pairs);
+  m.def("rope_pairs(Tensor src, Tensor(a!) dst, Tensor positions, Tensor rope, int half_dims) -> ()", &rope_pairs);
   m.def(
       "latent_attn(Tensor q, Tensor cache, Tensor block_tables, Tensor row_seq, Tensor positions, float scale, "
-      "int kv_rank, Tensor(a!) out, Tensor(b!)? part_o, Tensor(c!)? part_ml, Tensor? tiles, Tensor? cu_q, int impl) -> int",
+      "int kv_rank, Tensor(a!) out, Tensor(b!)? part_o, Tensor(c!)? part_ml, Tensor? tiles, Tensor? cu_q, int impl, "
+      "int window) -> int",
       &latent_attn);
   m.def("clamped_glu(Tensor gu, float limit, float alpha, Tensor(a!) out) -> ()", &clamped_glu);
   m.def("sigmoid_topk(Tensor x, Tensor Wr, int k, Tensor(a!) ids, Tensor(b!) w) -> ()", &sigmoid_topk);

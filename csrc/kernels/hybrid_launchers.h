@@ -77,6 +77,37 @@ void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* 
                     const void* shared, const void* sgate, long long ldsg, float* out, int T, int d, int f32,
                     hipStream_t s);
 
+// x[row] = table[token] * scale, token as for launch_embed_norm
+void launch_embed_scale(const int* ids, const int* src, const int* prev, const void* table, float scale, float* x, int T,
+                        int d, int f32, hipStream_t s);
+// ConvArgs with xin / state / w fp32 and no bias: out (activation dtype) = x + sum_j w[c][taps - 1 - j] x[t - j][c];
+// the carried taps are then stored by launch_conv_state_update(a, 1, s)
+void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s);
+// x = (alpha x + delta) / rms * w, in place on the fp32 stream (delta in the activation dtype)
+void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T, int d, int f32,
+                          hipStream_t s);
+// z[t] = q (H dk) | k (G dk) | v (G dv); q_out [T][H][dk] = q / rms_head * wq * q_mult[h]; cache rows `slot` (>= 0):
+// k_cache [rows][G][dk] = k / rms_head * wk, v_cache [rows][G][dv] = v
+struct QkNormArgs {
+  const void* z; long long ldz;
+  int H, G, dk, dv;
+  const float* wq;      // [dk]
+  const float* wk;      // [dk]
+  const float* q_mult;  // [H] or null
+  float eps;
+  const int* slots;
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+};
+void launch_qk_norm_cache(const QkNormArgs& a, int T, int f32, hipStream_t s);
+// out = gelu_tanh(gate) * up
+void launch_gelu_tanh_mul(const void* gate, long long ldg, const void* up, long long ldu, void* out, int R, int F, int f32,
+                          hipStream_t s);
+// out = a * sigmoid(gate) (out may be a)
+void launch_sigmoid_mul(const void* a, long long lda, const void* gate, long long ldg, void* out, int R, int F, int f32,
+                        hipStream_t s);
+
 // ---- window_attention.hip ------------------------------------------------------------------------------
 struct WindowAttnArgs {
   const void* q;        // [T][H][dk]
@@ -87,6 +118,7 @@ struct WindowAttnArgs {
   const int* positions; // [T]: row sees positions max(0, p - window + 1) .. p
   const void* gate;     // [T][H] (row stride ldg) or null: output times sigmoid(gate)
   long long ldg;
+  const float* bias;    // [2][H] or null: score of a key at distance n lowered by bias[0][h] * ln(1 + bias[1][h] * n)
   void* out;            // [T][H][dv]
   int T, H, G, dk, dv, BS, max_blocks, window;
   int bs_shift;         // log2(BS), or -1 if BS is no power of two (set by the launcher)

@@ -11,6 +11,11 @@
 //   relu_sq, silu_mul   feed-forward activations on column ranges of a fused projection
 //   softmax_topk        router: fp32 softmax over all outputs, choice by score + correction, weights = plain scores
 //   moe_mix             weighted sum of the chosen experts' rows (identity experts: the input row) + gated shared expert
+//   embed_scale         x = table[token] * scale                            (fp32 stream)
+//   residual_conv       sublayer input x + causal per-channel convolution of the fp32 stream, carried taps fp32
+//   post_rms_norm       norm after the sum: x = rms_norm(alpha x + delta) * w, in place on the fp32 stream
+//   qk_norm_cache       per-head RMS norm of queries (times a per-head factor) and keys, paged key / value cache write
+//   gelu_tanh_mul, sigmoid_mul   gated activations on column ranges of a fused projection
 //
 // One workgroup per row unless noted; columns strided over the threads (coalesced), any width.  All statistics,
 // rotations, gates and sums are fp32; only the stored activations take the activation dtype T (bf16 or float).
@@ -285,6 +290,126 @@ __global__ __launch_bounds__(NT) void moe_mix_kernel(const T* __restrict__ y, co
   }
 }
 
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void embed_scale_kernel(const int* __restrict__ ids, const int* __restrict__ src,
+                                                         const int* __restrict__ prev, const T* __restrict__ table,
+                                                         float scale, float* __restrict__ x, int d) {
+  const int row = blockIdx.x;
+  const int sr = src ? src[row] : -1;
+  const long long tok = sr >= 0 ? prev[sr] : ids[row];
+  const T* t = table + tok * d;
+  for (int c = threadIdx.x; c < d; c += BT) x[(long long)row * d + c] = (float)t[c] * scale;
+}
+
+// grid (T, ceil(C / NT)): one thread per (row, channel).  x and the carried taps are fp32, the output takes the
+// activation dtype: out = x + sum_i w[c][taps - 1 - i] x[t - i][c]
+template <typename T>
+__global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
+  const int row = blockIdx.x, c = blockIdx.y * NT + threadIdx.x;
+  if (c >= a.C) return;
+  const int s0 = a.cu_q ? a.cu_q[a.row_seq[row]] : row;
+  const int j = row - s0, taps = a.taps;
+  const int pr = a.prev_row[s0];
+  const float* st = pr <= -2 ? reinterpret_cast<const float*>(a.state) + (long long)(-(pr + 2)) * a.state_stride : nullptr;
+  const float* x = reinterpret_cast<const float*>(a.xin);
+  const float* w = reinterpret_cast<const float*>(a.w) + (long long)c * taps;
+  float acc = x[(long long)row * a.ldx + c];
+  for (int i = 0; i < taps; ++i) {       // i positions back
+    float v = 0.f;
+    if (i <= j) v = x[(long long)(row - i) * a.ldx + c];
+    else if (st) v = st[(long long)(taps - 1 - (i - j)) * a.C + c];
+    acc += w[taps - 1 - i] * v;
+  }
+  reinterpret_cast<T*>(a.out)[(long long)row * a.C + c] = (T)acc;
+}
+
+// one workgroup per row; the row's sums stay in registers between the two passes (up to PER columns per thread, wider
+// rows recompute)
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void post_rms_norm_kernel(float* __restrict__ x, float alpha, const T* __restrict__ delta,
+                                                           const float* __restrict__ w, float eps, int d) {
+  __shared__ float scratch[BT / 64];
+  constexpr int PER = 8;
+  const long long o = (long long)blockIdx.x * d;
+  float v[PER];
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * BT;
+    v[i] = c < d ? alpha * x[o + c] + (float)delta[o + c] : 0.f;
+    sq += v[i] * v[i];
+  }
+  for (int c = threadIdx.x + PER * BT; c < d; c += BT) {
+    const float u = alpha * x[o + c] + (float)delta[o + c];
+    sq += u * u;
+  }
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
+  // (each thread rewrites only the columns it read itself)
+  for (int c = threadIdx.x + PER * BT; c < d; c += BT) x[o + c] = (alpha * x[o + c] + (float)delta[o + c]) * r * w[c];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * BT;
+    if (c < d) x[o + c] = v[i] * r * w[c];
+  }
+}
+
+// grid (T, ceil((H + G) / 4)), 4 waves: one wave per query or key head normalises it (lanes over the head's entries);
+// the workgroups then copy the value heads in strides.
+template <typename T>
+__global__ __launch_bounds__(NT) void qk_norm_cache_kernel(QkNormArgs a) {
+  const int row = blockIdx.x, lane = threadIdx.x & 63;
+  const int head = blockIdx.y * (NT / 64) + (threadIdx.x >> 6);
+  const T* z = reinterpret_cast<const T*>(a.z) + (long long)row * a.ldz;
+  const int slot = a.slots[row];
+  const int nq = a.H * a.dk, nk = a.G * a.dk, nv = a.G * a.dv;
+  if (head < a.H + a.G) {
+    const bool isq = head < a.H;
+    const T* src = z + (long long)head * a.dk;           // query heads, then key heads, contiguous
+    float sq = 0.f;
+    for (int e = lane; e < a.dk; e += 64) {
+      const float v = (float)src[e];
+      sq += v * v;
+    }
+    float r = 1.f / sqrtf(wave_sum(sq) / (float)a.dk + a.eps);
+    const float* w = isq ? a.wq : a.wk;
+    T* dst = nullptr;
+    if (isq) {
+      dst = reinterpret_cast<T*>(a.q_out) + ((long long)row * a.H + head) * a.dk;
+      if (a.q_mult) r *= a.q_mult[head];
+    } else if (slot >= 0) {
+      dst = reinterpret_cast<T*>(a.k_cache) + ((long long)slot * a.G + (head - a.H)) * a.dk;
+    }
+    if (dst)
+      for (int e = lane; e < a.dk; e += 64) dst[e] = (T)((float)src[e] * w[e] * r);
+  }
+  if (slot >= 0) {
+    T* vc = reinterpret_cast<T*>(a.v_cache) + (long long)slot * nv;
+    for (int i = blockIdx.y * NT + threadIdx.x; i < nv; i += gridDim.y * NT) vc[i] = z[nq + nk + i];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void gelu_tanh_mul_kernel(const T* __restrict__ g, long long ldg, const T* __restrict__ u,
+                                                           long long ldu, T* __restrict__ out, int R, int F) {
+  const long long n = (long long)R * F;
+  for (long long i = (long long)blockIdx.x * NT + threadIdx.x; i < n; i += (long long)gridDim.x * NT) {
+    const long long r = i / F, c = i - r * F;
+    const float gv = (float)g[r * ldg + c];
+    const float t = tanhf(0.7978845608028654f * (gv + 0.044715f * gv * gv * gv));
+    out[i] = (T)(0.5f * gv * (1.f + t) * (float)u[r * ldu + c]);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void sigmoid_mul_kernel(const T* a, long long lda, const T* __restrict__ g,
+                                                         long long ldg, T* out, int R, int F) {
+  const long long n = (long long)R * F;
+  for (long long i = (long long)blockIdx.x * NT + threadIdx.x; i < n; i += (long long)gridDim.x * NT) {
+    const long long r = i / F, c = i - r * F;
+    out[i] = (T)((float)a[r * lda + c] * sigmoidf((float)g[r * ldg + c]));
+  }
+}
+
 int ew_grid(long long n) {
   long long g = (n + NT - 1) / NT;
   return (int)(g < 1 ? 1 : (g > 16384 ? 16384 : g));
@@ -395,4 +520,50 @@ void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* 
   if (T_ <= 0) return;
   DISPATCH_T(f32, moe_mix_kernel<T><<<T_, NT, 0, s>>>((const T*)y, dst, ids, w, k, E, (const T*)h, (const T*)shared,
                                                      (const T*)sgate, ldsg, out, d);)
+}
+
+void launch_embed_scale(const int* ids, const int* src, const int* prev, const void* table, float scale, float* x, int T_,
+                        int d, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  if (wide_rows(T_, d)) {
+    DISPATCH_T(f32, (embed_scale_kernel<T, 1024><<<T_, 1024, 0, s>>>(ids, src, prev, (const T*)table, scale, x, d));)
+  } else {
+    DISPATCH_T(f32, (embed_scale_kernel<T, NT><<<T_, NT, 0, s>>>(ids, src, prev, (const T*)table, scale, x, d));)
+  }
+}
+
+void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s) {
+  if (a.T <= 0) return;
+  dim3 grid(a.T, (a.C + NT - 1) / NT);
+  DISPATCH_T(f32, residual_conv_kernel<T><<<grid, NT, 0, s>>>(a);)
+}
+
+void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T_, int d, int f32,
+                          hipStream_t s) {
+  if (T_ <= 0) return;
+  if (wide_rows(T_, d)) {
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
+  } else {
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, NT><<<T_, NT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
+  }
+}
+
+void launch_qk_norm_cache(const QkNormArgs& a, int T_, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  dim3 grid(T_, (a.H + a.G + NT / 64 - 1) / (NT / 64));
+  DISPATCH_T(f32, qk_norm_cache_kernel<T><<<grid, NT, 0, s>>>(a);)
+}
+
+void launch_gelu_tanh_mul(const void* gate, long long ldg, const void* up, long long ldu, void* out, int R, int F, int f32,
+                          hipStream_t s) {
+  if (R <= 0) return;
+  DISPATCH_T(f32, gelu_tanh_mul_kernel<T><<<ew_grid((long long)R * F), NT, 0, s>>>((const T*)gate, ldg, (const T*)up,
+                                                                                   ldu, (T*)out, R, F);)
+}
+
+void launch_sigmoid_mul(const void* a, long long lda, const void* gate, long long ldg, void* out, int R, int F, int f32,
+                        hipStream_t s) {
+  if (R <= 0) return;
+  DISPATCH_T(f32, sigmoid_mul_kernel<T><<<ew_grid((long long)R * F), NT, 0, s>>>((const T*)a, lda, (const T*)gate, ldg,
+                                                                                 (T*)out, R, F);)
 }

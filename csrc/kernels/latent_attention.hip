@@ -12,8 +12,10 @@
 //
 //   latent_prep   per token: RMS-norm the query latent; RMS-norm the kv latent and rotate the shared key part into
 //                 the token's cache row (statistics and angles in fp32)
-//   rope_pairs    interleaved-pair rotary (dimension 2i with 2i + 1) of a strided [T][H][rot] slice
-//   latent_attn   causal softmax attention over the paged latent cache; scores, weights and accumulators fp32.
+//   rope_pairs    rotary of a strided [T][H][rot] slice: interleaved pairs (dimension 2i with 2i + 1) or the half
+//                 layout (dimension i with i + dims / 2, dimensions past dims passing)
+//   latent_attn   causal softmax attention over the paged latent cache, optionally limited to a sliding window of
+//                 the newest keys; scores, weights and accumulators fp32.
 //                 Two implementations: the MFMA kernel (bf16, tiled shapes) and a one-wave-per-(row, head) kernel
 //                 for every other shape and for the 32-bit model.
 //
@@ -33,6 +35,19 @@
 namespace {
 
 constexpr int NT = 256;
+
+// entries (first, second) of rotary pair p in a vector of `rot` entries.  Interleaved (half_dims == 0): (2p, 2p + 1).
+// Half layout: pair p < half_dims / 2 is (p, p + half_dims / 2); the pairs after those are the passing entries
+// half_dims .., two by two (their table entries are the identity).
+SYM_DEV void pair_entries(int p, int half_dims, int& e0, int& e1) {
+  if (half_dims == 0) {
+    e0 = 2 * p, e1 = 2 * p + 1;
+  } else if (p < half_dims / 2) {
+    e0 = p, e1 = p + half_dims / 2;
+  } else {
+    e0 = half_dims + 2 * (p - half_dims / 2), e1 = e0 + 1;
+  }
+}
 
 template <typename T>
 __global__ __launch_bounds__(NT) void latent_prep_kernel(LatentPrepArgs a) {
@@ -63,10 +78,12 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(LatentPrepArgs a) {
   for (int c = threadIdx.x; c < a.kv_rank; c += NT) out[c] = (T)((float)zk[c] * rk * (float)wkv[c]);
   const float* cs = a.rope + (long long)a.positions[row] * a.rot;
   for (int i = threadIdx.x; i < a.rot / 2; i += NT) {
-    const float u = (float)zk[a.kv_rank + 2 * i], v = (float)zk[a.kv_rank + 2 * i + 1];
+    int e0, e1;
+    pair_entries(i, a.half_dims, e0, e1);
+    const float u = (float)zk[a.kv_rank + e0], v = (float)zk[a.kv_rank + e1];
     const float co = cs[2 * i], si = cs[2 * i + 1];
-    out[a.kv_rank + 2 * i] = (T)(u * co - v * si);
-    out[a.kv_rank + 2 * i + 1] = (T)(v * co + u * si);
+    out[a.kv_rank + e0] = (T)(u * co - v * si);
+    out[a.kv_rank + e1] = (T)(v * co + u * si);
   }
 }
 
@@ -74,18 +91,21 @@ template <typename T>
 __global__ __launch_bounds__(NT) void rope_pairs_kernel(const T* __restrict__ src, long long s_t, long long s_h,
                                                         T* __restrict__ dst, long long d_t, long long d_h,
                                                         const int* __restrict__ positions,
-                                                        const float* __restrict__ rope, int H, int rot) {
+                                                        const float* __restrict__ rope, int H, int rot,
+                                                        int half_dims) {
   const int row = blockIdx.x;
   const float* cs = rope + (long long)positions[row] * rot;
   const int half = rot / 2;
   for (int i = threadIdx.x; i < H * half; i += NT) {
     const int h = i / half, p = i - h * half;
-    const T* s = src + row * s_t + h * s_h + 2 * p;
-    T* o = dst + row * d_t + h * d_h + 2 * p;
-    const float u = (float)s[0], v = (float)s[1];
+    int e0, e1;
+    pair_entries(p, half_dims, e0, e1);
+    const T* s = src + row * s_t + h * s_h;
+    T* o = dst + row * d_t + h * d_h;
+    const float u = (float)s[e0], v = (float)s[e1];
     const float co = cs[2 * p], si = cs[2 * p + 1];
-    o[0] = (T)(u * co - v * si);
-    o[1] = (T)(v * co + u * si);
+    o[e0] = (T)(u * co - v * si);
+    o[e1] = (T)(v * co + u * si);
   }
 }
 
@@ -130,7 +150,8 @@ __global__ __launch_bounds__(64) void latent_attn_wave_kernel(LatentAttnArgs a) 
   const int row = blockIdx.x, h = blockIdx.y, part = blockIdx.z;
   const int lane = threadIdx.x;
   const int nkeys = a.positions[row] + 1;
-  const int k0 = a.parts > 1 ? part * a.part_tokens : 0;
+  const int lo = a.window > 0 ? max(0, nkeys - a.window) : 0;     // the first key the row sees
+  const int k0 = a.parts > 1 ? lo + part * a.part_tokens : lo;
   const int k1 = a.parts > 1 ? min(nkeys, k0 + a.part_tokens) : nkeys;
   const T* q = (const T*)a.q + ((long long)row * a.H + h) * a.Dk;
   for (int c = lane; c < a.Dk; c += 64) qs[c] = (float)q[c];
@@ -150,7 +171,7 @@ __global__ __launch_bounds__(64) void latent_attn_wave_kernel(LatentAttnArgs a) 
       crow = bt[key / a.BS] * a.BS + key % a.BS;
       s = dot_row(qs, cache + (long long)crow * a.Dk, a.Dk) * a.scale;
     }
-    const float m_new = fmaxf(m, wave_max(s));
+    const float m_new = fmaxf(m, wave_max(s));   // finite: the tile holds at least one key the row sees
     const float alpha = expf(m - m_new);
     const float p = valid ? expf(s - m_new) : 0.f;
     l = l * alpha + wave_sum(p);
@@ -201,7 +222,9 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a
   __shared__ float stat[8];
   const int row = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const long long p0 = ((long long)row * a.H + h) * a.parts;
-  const int np = min(a.parts, (a.positions[row] + a.part_tokens) / a.part_tokens);  // partitions that hold keys
+  // partitions that hold keys: the row's range starts at its window's first key (at 0 without a window)
+  const int seen = a.window > 0 ? min(a.positions[row] + 1, a.window) : a.positions[row] + 1;
+  const int np = min(a.parts, (seen + a.part_tokens - 1) / a.part_tokens);
   float m = -INFINITY;
   for (int p = tid; p < np; p += 256) m = fmaxf(m, a.part_ml[2 * (p0 + p)]);
   m = wave_max(m);
@@ -282,7 +305,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     wave_active = blockIdx.y * 16 * QG + qg * 16 < H;
     limit = a.positions[qrow];
     part = blockIdx.z;
-    k_lo = a.parts > 1 ? part * a.part_tokens : 0;
+    const int first = a.window > 0 ? max(0, limit + 1 - a.window) : 0;
+    k_lo = a.parts > 1 ? first + part * a.part_tokens : first;
     k_hi = a.parts > 1 ? min(limit + 1, k_lo + a.part_tokens) : limit + 1;
     if (k_lo >= k_hi) return;  // a partition past this row's keys: the merge never reads it
     wave_hi = k_hi;
@@ -298,7 +322,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     qrow = q0 + min(rin, qlen - 1);
     head = blockIdx.y;
     limit = a.positions[qrow];
-    k_lo = 0;
+    k_lo = a.window > 0 ? max(0, a.positions[q0 + off] + 1 - a.window) : 0;   // the tile's first row looks back farthest
     k_hi = a.positions[q0 + min(off + 16 * QG - 1, qlen - 1)] + 1;       // a run's rows are consecutive positions
     wave_hi = a.positions[q0 + min(off + qg * 16 + 15, qlen - 1)] + 1;
     wave_lo = a.positions[q0 + min(off + qg * 16, qlen - 1)] + 1;
@@ -359,7 +383,9 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       if (k0 + 2 * KT < k_hi) fetch(k0 + 2 * KT, 0);
     }
     // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
-    const bool active = wave_active && k0 < wave_hi;  // (the same for the waves that share a query group)
+    // (the same for the waves that share a query group; with a window, a tile wholly before the first key of the wave's
+    // first row is seen by none of its rows)
+    const bool active = wave_active && k0 < wave_hi && (a.window <= 0 || k0 + KT > wave_lo - a.window);
     f32x4 st[2];
     if constexpr (DSPLIT == 2) {
       // the two waves of a query group each score one 16-key subtile (four accumulator chains over the k steps) and
@@ -405,7 +431,9 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       }
     }
     // scale; mask only where a tile reaches past some query vector's last key (the diagonal tiles, the range's tail)
-    const bool edge = k0 + KT > wave_lo || k0 + KT > k_hi;  // wave-uniform
+    // (wave-uniform; with a window also the tiles that start before the first key of the wave's last row)
+    const bool edge = k0 + KT > wave_lo || k0 + KT > k_hi || (a.window > 0 && k0 < wave_hi - a.window);
+    const int low = a.window > 0 ? limit + 1 - a.window : 0;  // this query vector's first key
     float mx = -INFINITY;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
@@ -414,7 +442,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
         float v = st[sub][i] * a.scale;
         if (edge) {
           const int key = k0 + sub * 16 + g * 4 + i;
-          if (key > limit || key >= k_hi) v = -INFINITY;
+          if (key > limit || key >= k_hi || key < low) v = -INFINITY;
         }
         st[sub][i] = v;
         mx = fmaxf(mx, v);
@@ -425,8 +453,10 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     // register) only when some query vector's maximum grew by more than 8; until then weights may reach e^8, which
     // fp32 sums and bf16 products hold as well as values below 1.  The first tile always takes the branch.
     if (__any(mx > m + 8.f)) {
-      const float m_new = fmaxf(m, mx);        // finite: every query vector sees the first key of its range
-      const float alpha = __expf(m - m_new);
+      // (without a window every query vector sees the first key of its range; with one, a vector may have seen nothing
+      // yet: its maximum stays -inf and nothing of it is rescaled)
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m_new == -INFINITY ? 1.f : __expf(m - m_new);
       l *= alpha;
 #pragma unroll
       for (int dt = 0; dt < RTD; ++dt)
@@ -439,7 +469,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = __expf(st[sub][i] - m);
+        const float p = m == -INFINITY ? 0.f : __expf(st[sub][i] - m);
         ps += p;
         pb.h[sub * 4 + i] = (bf16)p;
       }
@@ -544,12 +574,15 @@ void launch_latent_prep(const LatentPrepArgs& a, int T, int f32, hipStream_t s) 
 }
 
 void launch_rope_pairs(const void* src, long long s_t, long long s_h, void* dst, long long d_t, long long d_h,
-                       const int* positions, const float* rope, int T, int H, int rot, int f32, hipStream_t s) {
+                       const int* positions, const float* rope, int T, int H, int rot, int half_dims, int f32,
+                       hipStream_t s) {
   if (T <= 0 || rot <= 0) return;
   if (f32)
-    rope_pairs_kernel<float><<<T, NT, 0, s>>>((const float*)src, s_t, s_h, (float*)dst, d_t, d_h, positions, rope, H, rot);
+    rope_pairs_kernel<float><<<T, NT, 0, s>>>((const float*)src, s_t, s_h, (float*)dst, d_t, d_h, positions, rope, H, rot,
+                                              half_dims);
   else
-    rope_pairs_kernel<bf16><<<T, NT, 0, s>>>((const bf16*)src, s_t, s_h, (bf16*)dst, d_t, d_h, positions, rope, H, rot);
+    rope_pairs_kernel<bf16><<<T, NT, 0, s>>>((const bf16*)src, s_t, s_h, (bf16*)dst, d_t, d_h, positions, rope, H, rot,
+                                             half_dims);
 }
 
 int launch_latent_attn(const LatentAttnArgs& a, int f32, int impl, hipStream_t s) {

@@ -28,7 +28,8 @@ void launch_layer_norm(const float* x, const long long* rows, const void* w, flo
 // ---- latent_attention.hip ----------------------------------------------------------------------------
 struct LatentPrepArgs {
   const void* z;        // [T][nz] projections of the mixer input: q latent | kv latent | shared rotary key
-  int nz, q_rank, kv_rank, rot;  // kv_rank == 0: the layer has no kv part (it attends another layer's cache)
+  int nz, q_rank, kv_rank, rot;  // nz: row stride of z; kv_rank == 0: no kv part (the layer attends another's cache)
+  int half_dims;        // 0: rotary pairs (2i, 2i + 1); > 0: entry i pairs with i + half_dims / 2, later entries pass
   const void* wq;       // [q_rank] norm weight
   const void* wkv;      // [kv_rank]
   float eps;
@@ -39,21 +40,24 @@ struct LatentPrepArgs {
   void* cache;          // [rows][kv_rank + rot]
 };
 void launch_latent_prep(const LatentPrepArgs& a, int T, int f32, hipStream_t s);
-// interleaved-pair rotary of src[t][h][0..rot) -> dst[t][h][0..rot) (element strides given)
+// rotary of src[t][h][0..rot) -> dst[t][h][0..rot) (element strides given); half_dims as in LatentPrepArgs
 void launch_rope_pairs(const void* src, long long s_t, long long s_h, void* dst, long long d_t, long long d_h,
-                       const int* positions, const float* rope, int T, int H, int rot, int f32, hipStream_t s);
+                       const int* positions, const float* rope, int T, int H, int rot, int half_dims, int f32,
+                       hipStream_t s);
 struct LatentAttnArgs {
   const void* q;        // [T][H][Dk]: absorbed query (kv_rank) | rotated query (rot)
   const void* cache;    // [blocks][BS][Dk]
   const int* block_tables;  // [seqs][max_blocks]
   const int* row_seq;   // [T]
-  const int* positions; // [T]: a row sees keys 0..position
+  const int* positions; // [T]: a row sees keys 0..position (window > 0: position - window + 1..position)
+  int window;           // 0: no limit
   void* out;            // [T][H][kv_rank]: softmax-weighted sum of the latents
   float* part_o;        // split-KV partials (decode form): [T][H][parts][kv_rank], [T][H][parts][2]
   float* part_ml;
   int T, H, Dk, kv_rank, BS, max_blocks;
   int bs_shift;            // log2(BS), or -1 if BS is no power of two
-  int parts, part_tokens;  // split-KV: partition p of a row covers keys [p * part_tokens, (p + 1) * part_tokens)
+  int parts, part_tokens;  // split-KV: partition p of a row covers part_tokens keys from first + p * part_tokens on,
+                           // first = the row's first visible key
   float scale;
   // prompt form of the MFMA kernel: 64-row query tiles (sequence, first row within the sequence's run) over the
   // runs cu_q[seq] .. cu_q[seq + 1]; nullptr: one query row per sequence (decode steps)

@@ -1,5 +1,6 @@
 // Sliding-window softmax attention with grouped key / value heads over a paged cache, with an optional per-head
-// sigmoid output gate.
+// sigmoid output gate and an optional per-head logarithmic distance bias (the score of a key n positions back is
+// lowered by b1_h ln(1 + b2_h n)).
 //
 // Row r (position p of sequence row_seq[r]) sees positions max(0, p - window + 1) .. p; query head h reads key / value
 // head h / (H / G).  Key and value head sizes are independent (dk, dv).  Scores, softmax statistics, weights and the
@@ -79,9 +80,11 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
   const T* kc = reinterpret_cast<const T*>(a.k_cache);
   const T* vc = reinterpret_cast<const T*>(a.v_cache);
   float acc[REP][MAX_VCOLS];
-  float m[REP], l[REP];
+  float m[REP], l[REP], b1[REP], b2[REP];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
+    b1[r] = a.bias ? a.bias[h0 + r] : 0.f;
+    b2[r] = a.bias ? a.bias[a.H + h0 + r] : 0.f;
     m[r] = -INFINITY, l[r] = 0.f;
 #pragma unroll
     for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] = 0.f;
@@ -93,6 +96,11 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     if (j <= p) {
       slot = cache_row(bt, j, a.BS, a.bs_shift);
       dot_rows<T, REP>(kc + (slot * a.G + g) * a.dk, qs, a.dk, sc);
+      if (a.bias) {
+        const float dist = (float)(p - j);
+#pragma unroll
+        for (int r = 0; r < REP; ++r) sc[r] -= b1[r] * log1pf(b2[r] * dist);
+      }
     }
 #pragma unroll
     for (int r = 0; r < REP; ++r) {
@@ -246,6 +254,9 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
   for (int i = 0; i < VD; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const float sl2 = a.scale * 1.44269504088896341f;
+  // distance bias in units of log2(e): b1 ln(1 + b2 n) log2(e) = b1 log2(1 + b2 n)
+  const bool biased = a.bias != nullptr;
+  const float b1 = biased ? a.bias[h] : 0.f, b2 = biased ? a.bias[a.H + h] : 0.f;
   const int k_lo = max(0, p_first - a.window + 1);
   // cache blocks of 64 tokens or a multiple: a key tile lies in one block, whose number is read one tile ahead (the
   // rows' loads then do not wait for a block-table load of their own)
@@ -312,6 +323,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           pv[s4][e] = acc[e] * sl2;
+          if (biased) pv[s4][e] -= b1 * __log2f(1.f + b2 * (float)(qp - (kt + 16 * s4 + 4 * hq + e)));
           mx = fmaxf(mx, pv[s4][e]);
         }
       } else {
@@ -319,7 +331,9 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
         for (int e = 0; e < 4; ++e) {
           const int kp = kt + 16 * s4 + 4 * hq + e;
           const bool vis = rv && kp <= qp && kp > qp - a.window;
-          pv[s4][e] = vis ? acc[e] * sl2 : -INFINITY;
+          float sv = acc[e] * sl2;
+          if (biased) sv -= b1 * __log2f(1.f + b2 * (float)max(qp - kp, 0));
+          pv[s4][e] = vis ? sv : -INFINITY;
           mx = fmaxf(mx, pv[s4][e]);
         }
       }
