@@ -1,5 +1,6 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a Bozevik or Lemunex stack beside the closest Llama / Mixtral stack of equal size.
+"""Prefill and decode throughput of a Bozevik, Lemunex or Komazen stack beside the closest Llama / Mixtral stack of equal
+size.
 
 Random weights, layer shapes of real models, a few layers each (throughput per layer is what is compared; the
 vocabulary projection is the same size on both sides).  Per size and family, through the engine's own scheduler:
@@ -66,6 +67,23 @@ def _lemunex_pairs():
     }
 
 
+def _komazen_pairs():
+    """Komazen stacks (latent attention with a sliding window, one layer attending its neighbour's cache, between plain
+    grouped-head attention layers with the distance bias) beside the Llama stack of the same width, head count and
+    feed-forward width; the window equals the benchmark's prompt length."""
+    from symmetry_amd.models.config import ModelConfig, komazen_stack
+
+    kw = dict(max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+    return {
+        "w2048": (komazen_stack("komazen-w2048", 32768, 2048, "LASA", heads=16, kv_heads=4, dim=128, ff=8192, window=1024,
+                                embed_scale=8.0, postln_alpha=2.0, **kw),
+                  ModelConfig("llama-w2048", 32768, 2048, 8192, 4, 16, 4, **kw)),
+        "w4096": (komazen_stack("komazen-w4096", 32768, 4096, "LASA", heads=32, kv_heads=8, dim=128, ff=14336, window=1024,
+                                embed_scale=8.0, postln_alpha=2.0, **kw),
+                  ModelConfig("llama-w4096", 32768, 4096, 14336, 4, 32, 8, **kw)),
+    }
+
+
 def measure(mcfg, prompts: int, plen: int, steps: int, reps: int = 3) -> dict:
     import torch
 
@@ -117,12 +135,14 @@ def main(argv=None) -> int:
     ap.add_argument("--prompts", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--decode-steps", type=int, default=64)
-    ap.add_argument("--only", default="", help="bozevik | lemunex | baseline: one side only (profiling)")
-    ap.add_argument("--design", default="bozevik", choices=("bozevik", "lemunex"), help="the family measured")
+    ap.add_argument("--only", default="", help="bozevik | lemunex | komazen | baseline: one side only (profiling)")
+    ap.add_argument("--design", default="bozevik", choices=("bozevik", "lemunex", "komazen"), help="the family measured")
     a = ap.parse_args(argv)
-    pairs = _pairs() if a.design == "bozevik" else _lemunex_pairs()
+    pairs = {"bozevik": _pairs, "lemunex": _lemunex_pairs, "komazen": _komazen_pairs}[a.design]()
     ratios = {}
     for size in a.sizes.split(","):
+        if size not in pairs:     # (a design without routed layers has no routed size)
+            continue
         boz, base = pairs[size]
         rows = {}
         for side, cfg in ((a.design, boz), ("baseline", base)):

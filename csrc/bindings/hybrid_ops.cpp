@@ -467,13 +467,15 @@ void embed_scale(const Tensor& ids, const OptTensor& src, const OptTensor& prev,
 }
 
 void residual_conv(const Tensor& x, const Tensor& w, Tensor& state, const OptTensor& cu_q, const OptTensor& row_seq,
-                   const Tensor& prev_row, int64_t runs, Tensor& out) {
+                   const Tensor& prev_row, const OptTensor& save_slot, int64_t runs, Tensor& out) {
   const int f32 = act(out, "out");
   dtype(x, at::kFloat, "x");
   dtype(w, at::kFloat, "w");
   dtype(state, at::kFloat, "state");
-  ConvArgs a = conv_args(x, w, std::nullopt, state, cu_q, row_seq, prev_row, std::nullopt, runs, 1);
+  ConvArgs a = conv_args(x, w, std::nullopt, state, cu_q, row_seq, prev_row, save_slot, runs, 1);
   TORCH_CHECK(!cu_q.has_value() || row_seq.has_value(), "residual_conv: cu_q without row_seq");
+  TORCH_CHECK(!(cu_q.has_value() && save_slot.has_value()), "residual_conv: the taps move on in this launch only where "
+              "every row is a run of its own");
   TORCH_CHECK(out.numel() == (int64_t)a.T * a.C, "residual_conv: out shape");
   a.out = out.data_ptr();
   launch_residual_conv(a, f32, cur_stream(out));
@@ -587,7 +589,8 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
   m.def("grouped_linear(Tensor xs, Tensor W, Tensor offsets, Tensor(a!) y) -> ()", &grouped_linear);
   m.def("embed_scale(Tensor ids, Tensor? src, Tensor? prev, Tensor table, float scale, Tensor(a!) x) -> ()", &embed_scale);
   m.def(
-      "residual_conv(Tensor x, Tensor w, Tensor(a!) state, Tensor? cu_q, Tensor? row_seq, Tensor prev_row, int runs, "
+      "residual_conv(Tensor x, Tensor w, Tensor(a!) state, Tensor? cu_q, Tensor? row_seq, Tensor prev_row, "
+      "Tensor? save_slot, int runs, "
       "Tensor(b!) out) -> ()",
       &residual_conv);
   m.def("post_rms_norm(Tensor(a!) x, float alpha, Tensor delta, Tensor w, float eps) -> ()", &post_rms_norm);

@@ -81,7 +81,8 @@ void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* 
 void launch_embed_scale(const int* ids, const int* src, const int* prev, const void* table, float scale, float* x, int T,
                         int d, int f32, hipStream_t s);
 // ConvArgs with xin / state / w fp32 and no bias: out (activation dtype) = x + sum_j w[c][taps - 1 - j] x[t - j][c];
-// the carried taps are then stored by launch_conv_state_update(a, 1, s)
+// the carried taps are then stored by launch_conv_state_update(a, 1, s) -- or by this launch itself where every row is a
+// run of its own (cu_q null) and save_slot is given
 void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s);
 // x = (alpha x + delta) / rms * w, in place on the fp32 stream (delta in the activation dtype)
 void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T, int d, int f32,

@@ -321,6 +321,21 @@ __global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
     acc += w[taps - 1 - i] * v;
   }
   reinterpret_cast<T*>(a.out)[(long long)row * a.C + c] = (T)acc;
+  // rows that are runs of their own (decode steps): this thread alone reads and writes its channel of the row's slot, so
+  // the carried taps move on here (older ones one place down, the row's input on top)
+  if (!a.cu_q && a.save_slot && taps > 1) {
+    const int sv = a.save_slot[row];
+    if (sv < 0) return;
+    const int keep = taps - 1;
+    float vals[MAX_TAPS];
+#pragma unroll
+    for (int m = 0; m < MAX_TAPS; ++m)
+      if (m < keep) vals[m] = m + 1 < keep ? (st ? st[(long long)(m + 1) * a.C + c] : 0.f) : x[(long long)row * a.ldx + c];
+    float* dst = reinterpret_cast<float*>(a.state) + (long long)sv * a.state_stride;
+#pragma unroll
+    for (int m = 0; m < MAX_TAPS; ++m)
+      if (m < keep) dst[(long long)m * a.C + c] = vals[m];
+  }
 }
 
 // one workgroup per row; the row's sums stay in registers between the two passes (up to PER columns per thread, wider

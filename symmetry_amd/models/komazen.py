@@ -184,10 +184,12 @@ class KomazenLM:
 
     def _conv(self, b: ForwardBatch, x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, runs: int) -> torch.Tensor:
         """The sublayer input x + conv(x) in the activation dtype; the run's newest rows of x become the carried taps."""
-        cu = b.cu_q if b.kind != "decode" else None
         h = self._buf("h", x.shape)
-        ops.residual_conv(x, w, state, cu, b.row_seq, b.prev_row, runs, h)
-        ops.conv_state_update(x, state, cu, b.prev_row, b.save_slot, runs)
+        if b.kind == "decode":      # every row a run of its own: one launch convolves and moves the carried taps on
+            ops.residual_conv(x, w, state, None, b.row_seq, b.prev_row, runs, h, save_slot=b.save_slot)
+        else:
+            ops.residual_conv(x, w, state, b.cu_q, b.row_seq, b.prev_row, runs, h)
+            ops.conv_state_update(x, state, b.cu_q, b.prev_row, b.save_slot, runs)
         return h
 
     def _latent(self, P: dict, b: ForwardBatch, cache: KomazenCache, h: torch.Tensor) -> torch.Tensor:

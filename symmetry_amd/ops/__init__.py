@@ -875,13 +875,19 @@ def embed_scale(ids, table, scale, x, src=None, prev=None):
     return reference.embed_scale(reference.resolve_ids(ids, src, prev), table, scale, x)
 
 
-def residual_conv(x, w, state, cu_q, row_seq, prev_row, runs, out):
+def residual_conv(x, w, state, cu_q, row_seq, prev_row, runs, out, save_slot=None):
     """out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j) per channel over every run of rows of the fp32 stream x (the
     sublayer input in the activation dtype); inputs before the run come from state[slot] [taps - 1, C] fp32
-    (prev_row[first] <= -2) or are zero.  ``conv_state_update(x, state, ...)`` then stores the run's newest inputs."""
+    (prev_row[first] <= -2) or are zero.  ``conv_state_update(x, state, ...)`` then stores the run's newest inputs; where
+    every row is a run of its own (cu_q None: decode steps), ``save_slot`` makes this launch store them itself."""
+    if save_slot is not None and cu_q is not None:
+        raise ValueError("residual_conv: save_slot only where every row is a run of its own")
     if _gpu(out):
-        return _hyb().residual_conv(x, w, state, cu_q, row_seq if cu_q is not None else None, prev_row, int(runs), out)
-    return reference.residual_conv(x, w, state, cu_q, prev_row, runs, out)
+        return _hyb().residual_conv(x, w, state, cu_q, row_seq if cu_q is not None else None, prev_row, save_slot,
+                                    int(runs), out)
+    reference.residual_conv(x, w, state, cu_q, prev_row, runs, out)
+    if save_slot is not None:
+        reference.conv_state_update(x, state, cu_q, prev_row, save_slot, runs)
 
 
 def post_rms_norm(x, alpha, delta, w, eps):
