@@ -481,13 +481,35 @@ void residual_conv(const Tensor& x, const Tensor& w, Tensor& state, const OptTen
   launch_residual_conv(a, f32, cur_stream(out));
 }
 
-void post_rms_norm(Tensor& x, double alpha, const Tensor& delta, const Tensor& w, double eps) {
+void post_rms_norm(Tensor& x, double alpha, const Tensor& delta, const Tensor& w, double eps, const OptTensor& conv_w,
+                   OptTensor conv_state, const OptTensor& prev_row, const OptTensor& save_slot, OptTensor h) {
   const int f32 = act(delta, "delta");
   dtype(x, at::kFloat, "x");
   dtype(w, at::kFloat, "w");
   TORCH_CHECK(x.dim() == 2 && delta.numel() == x.numel() && w.numel() == x.size(1), "post_rms_norm: x [T, d], delta [T, d]");
-  launch_post_rms_norm(ptr<float>(x), (float)alpha, delta.data_ptr(), ptr<float>(w), (float)eps, (int)x.size(0),
-                       (int)x.size(1), f32, cur_stream(x));
+  const int64_t T = x.size(0), d = x.size(1);
+  NormConvArgs cv{};
+  if (h.has_value()) {
+    TORCH_CHECK(conv_w.has_value() && conv_state.has_value() && prev_row.has_value() && save_slot.has_value(),
+                "post_rms_norm: the convolution needs its taps, state, prev_row and save_slot");
+    same_act(*h, f32, "h");
+    dtype(*conv_w, at::kFloat, "conv_w");
+    dtype(*conv_state, at::kFloat, "conv_state");
+    dtype(*prev_row, at::kInt, "prev_row");
+    dtype(*save_slot, at::kInt, "save_slot");
+    TORCH_CHECK(conv_w->dim() == 2 && conv_w->size(0) == d && conv_state->dim() == 3 && conv_state->size(2) == d &&
+                    conv_state->size(1) + 1 == conv_w->size(1) && conv_w->size(1) <= 16 && h->numel() == T * d &&
+                    prev_row->numel() >= T && save_slot->numel() >= T, "post_rms_norm: convolution shapes");
+    cv.w = ptr<float>(*conv_w);
+    cv.state = ptr<float>(*conv_state);
+    cv.state_stride = conv_state->stride(0);
+    cv.prev_row = ptr<int>(*prev_row);
+    cv.save_slot = ptr<int>(*save_slot);
+    cv.h = h->data_ptr();
+    cv.taps = (int)conv_w->size(1);
+  }
+  launch_post_rms_norm(ptr<float>(x), (float)alpha, delta.data_ptr(), ptr<float>(w), (float)eps, (int)T, (int)d, cv, f32,
+                       cur_stream(x));
 }
 
 void qk_norm_cache(const Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const Tensor& wq, const Tensor& wk,
@@ -593,7 +615,10 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
       "Tensor? save_slot, int runs, "
       "Tensor(b!) out) -> ()",
       &residual_conv);
-  m.def("post_rms_norm(Tensor(a!) x, float alpha, Tensor delta, Tensor w, float eps) -> ()", &post_rms_norm);
+  m.def(
+      "post_rms_norm(Tensor(a!) x, float alpha, Tensor delta, Tensor w, float eps, Tensor? conv_w, Tensor(b!)? conv_state, "
+      "Tensor? prev_row, Tensor? save_slot, Tensor(c!)? h) -> ()",
+      &post_rms_norm);
   m.def(
       "qk_norm_cache(Tensor z, int H, int G, int dk, int dv, Tensor wq, Tensor wk, Tensor? q_mult, float eps, Tensor slots, "
       "Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()",

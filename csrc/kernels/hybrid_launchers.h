@@ -84,9 +84,19 @@ void launch_embed_scale(const int* ids, const int* src, const int* prev, const v
 // the carried taps are then stored by launch_conv_state_update(a, 1, s) -- or by this launch itself where every row is a
 // run of its own (cu_q null) and save_slot is given
 void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s);
-// x = (alpha x + delta) / rms * w, in place on the fp32 stream (delta in the activation dtype)
-void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T, int d, int f32,
-                          hipStream_t s);
+// x = (alpha x + delta) / rms * w, in place on the fp32 stream (delta in the activation dtype).  With cv.h set (every row
+// a run of its own): also h = x_new + conv(x_new) over the row's carried taps (as launch_residual_conv), which move on
+struct NormConvArgs {
+  const float* w;        // [d][taps]
+  float* state;          // [slots][taps - 1][d]
+  long long state_stride;
+  const int* prev_row;
+  const int* save_slot;
+  void* h;               // [T][d] activation dtype, or null: no convolution
+  int taps;
+};
+void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T, int d,
+                          const NormConvArgs& cv, int f32, hipStream_t s);
 // z[t] = q (H dk) | k (G dk) | v (G dv); q_out [T][H][dk] = q / rms_head * wq * q_mult[h]; cache rows `slot` (>= 0):
 // k_cache [rows][G][dk] = k / rms_head * wk, v_cache [rows][G][dv] = v
 struct QkNormArgs {

@@ -339,13 +339,16 @@ __global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
 }
 
 // one workgroup per row; the row's sums stay in registers between the two passes (up to PER columns per thread, wider
-// rows recompute)
+// rows recompute).  With `cv` (rows that are runs of their own: decode steps) the same launch also makes the next
+// sublayer's input h = x_new + conv(x_new) from the row's carried taps and moves the taps on: a thread owns its columns
+// of the row and of the row's slot.
 template <typename T, int BT>
 __global__ __launch_bounds__(BT) void post_rms_norm_kernel(float* __restrict__ x, float alpha, const T* __restrict__ delta,
-                                                           const float* __restrict__ w, float eps, int d) {
+                                                           const float* __restrict__ w, float eps, int d, NormConvArgs cv) {
   __shared__ float scratch[BT / 64];
   constexpr int PER = 8;
-  const long long o = (long long)blockIdx.x * d;
+  const int row = blockIdx.x;
+  const long long o = (long long)row * d;
   float v[PER];
   float sq = 0.f;
 #pragma unroll
@@ -359,12 +362,39 @@ __global__ __launch_bounds__(BT) void post_rms_norm_kernel(float* __restrict__ x
     sq += u * u;
   }
   const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
+  const float* st = nullptr;
+  float* dst = nullptr;
+  if (cv.h) {
+    const int pr = cv.prev_row[row], sv = cv.save_slot[row];
+    if (pr <= -2) st = cv.state + (long long)(-(pr + 2)) * cv.state_stride;
+    if (sv >= 0) dst = cv.state + (long long)sv * cv.state_stride;
+  }
+  auto finish = [&](int c, float xn) {
+    x[o + c] = xn;
+    if (!cv.h) return;
+    const int taps = cv.taps, keep = taps - 1;
+    const float* cw = cv.w + (long long)c * taps;
+    float old[MAX_TAPS];
+    float acc = xn + cw[keep] * xn;
+#pragma unroll
+    for (int m = 0; m < MAX_TAPS; ++m)
+      if (m < keep) {
+        old[m] = st ? st[(long long)m * d + c] : 0.f;     // old[m]: the input keep - m positions back
+        acc += cw[m] * old[m];
+      }
+    reinterpret_cast<T*>(cv.h)[o + c] = (T)acc;
+    if (dst) {
+#pragma unroll
+      for (int m = 0; m < MAX_TAPS; ++m)
+        if (m < keep) dst[(long long)m * d + c] = m + 1 < keep ? old[m + 1] : xn;
+    }
+  };
   // (each thread rewrites only the columns it read itself)
-  for (int c = threadIdx.x + PER * BT; c < d; c += BT) x[o + c] = (alpha * x[o + c] + (float)delta[o + c]) * r * w[c];
+  for (int c = threadIdx.x + PER * BT; c < d; c += BT) finish(c, (alpha * x[o + c] + (float)delta[o + c]) * r * w[c]);
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int c = threadIdx.x + i * BT;
-    if (c < d) x[o + c] = v[i] * r * w[c];
+    if (c < d) finish(c, v[i] * r * w[c]);
   }
 }
 
@@ -553,13 +583,13 @@ void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s) {
   DISPATCH_T(f32, residual_conv_kernel<T><<<grid, NT, 0, s>>>(a);)
 }
 
-void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T_, int d, int f32,
-                          hipStream_t s) {
+void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T_, int d,
+                          const NormConvArgs& cv, int f32, hipStream_t s) {
   if (T_ <= 0) return;
   if (wide_rows(T_, d)) {
-    DISPATCH_T(f32, (post_rms_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv));)
   } else {
-    DISPATCH_T(f32, (post_rms_norm_kernel<T, NT><<<T_, NT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, NT><<<T_, NT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv));)
   }
 }
 

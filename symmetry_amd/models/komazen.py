@@ -20,10 +20,12 @@ v / sqrt(mean(v^2) + eps) * g; c(v) = v + a causal per-channel convolution of v 
     ff: W_down (gelu_tanh(W_gate h) * W_up h)
 
 Every projection that reads a sublayer's input is one row block of one fused weight (a single library GEMM); the
-kernels take column ranges of its output as views.  Step launches per layer: residual_conv, conv_state_update, GEMM,
+kernels take column ranges of its output as views.  Step launches per layer: GEMM (the mixer's projections),
 then latent: latent_prep, GEMM W_uq, bmm (absorb W_uk), rope_pairs, latent_attn, bmm (W_uv), sigmoid_mul, GEMM W_o
      plain:  qk_norm_cache, window_attn (distance bias), GEMM W_o
-post_rms_norm; residual_conv, conv_state_update, GEMM gate|up, gelu_tanh_mul, GEMM down, post_rms_norm.
+post_rms_norm, residual_conv, conv_state_update; GEMM gate|up, gelu_tanh_mul, GEMM down; post_rms_norm, residual_conv,
+conv_state_update (the next layer's input).  In decode steps every row is a run of its own, and one post_rms_norm launch
+norms the stream, convolves with the row's carried taps and moves them on.
 All intermediates live in the preallocated Workspace, so decode steps are hipGraph-capturable.
 
 fp32 in both serving dtypes: the stream, the convolutions' carried inputs, norm statistics, rotary angles, attention
@@ -192,6 +194,20 @@ class KomazenLM:
             ops.conv_state_update(x, state, b.cu_q, b.prev_row, b.save_slot, runs)
         return h
 
+    def _norm_conv(self, b: ForwardBatch, x: torch.Tensor, delta: torch.Tensor, w: torch.Tensor, conv, runs: int):
+        """x <- n(alpha x + delta, w); then the next sublayer's input from ``conv`` = (taps, carried state), if there is
+        one.  In decode steps one launch does both (a row is a run of its own there)."""
+        alpha, eps = self.cfg.postln_alpha, self.cfg.norm_eps
+        if conv is None:
+            ops.post_rms_norm(x, alpha, delta, w, eps)
+            return None
+        if b.kind == "decode":
+            h = self._buf("h", x.shape)
+            ops.post_rms_norm(x, alpha, delta, w, eps, conv[0], conv[1], b.prev_row, b.save_slot, h)
+            return h
+        ops.post_rms_norm(x, alpha, delta, w, eps)
+        return self._conv(b, x, conv[0], conv[1], runs)
+
     def _latent(self, P: dict, b: ForwardBatch, cache: KomazenCache, h: torch.Tensor) -> torch.Tensor:
         m = P["mixer"]
         T, H, r, rot, dn = h.shape[0], m.heads, m.kv_rank, m.rot_dim, m.dim
@@ -245,18 +261,20 @@ class KomazenLM:
         x = self._buf("x", (T, d), torch.float32)
         src = b.src if b.src is not None and b.kind == "decode" else None
         ops.embed_scale(b.input_ids, self.embed, cfg.embed_scale, x, src, self.last_ids if src is not None else None)
+        h = self._conv(b, x, self.L[0]["canon1"], cache.conv[0], runs)
         for i, P in enumerate(self.L):
-            h = self._conv(b, x, P["canon1"], cache.conv[2 * i], runs)
             att = self._latent(P, b, cache, h) if P["kind"] == "latent_attention" else self._attention(i, P, b, cache, h)
-            ops.post_rms_norm(x, alpha, att, P["norm1"], eps)
+            nxt = self.L[i + 1] if i + 1 < len(self.L) else None
+            after = (nxt["canon1"], cache.conv[2 * i + 2]) if nxt is not None else None
             if P["mlp"] is None:
+                h = self._norm_conv(b, x, att, P["norm1"], after, runs)
                 continue
-            h = self._conv(b, x, P["canon2"], cache.conv[2 * i + 1], runs)
+            h = self._norm_conv(b, x, att, P["norm1"], (P["canon2"], cache.conv[2 * i + 1]), runs)
             F = P["mlp"].ff
             gu = self._linear("ff.gu", h, P["w_gu"])
             act = self._buf("ff.act", (T, F))
             ops.gelu_tanh_mul(gu[:, :F], gu[:, F:], act)
-            ops.post_rms_norm(x, alpha, self._linear("ff.down", act, P["w_down"]), P["norm2"], eps)
+            h = self._norm_conv(b, x, self._linear("ff.down", act, P["w_down"]), P["norm2"], after, runs)
         n = b.num_seqs
         ids = self.last_ids[:n]
         self.last_logits = None

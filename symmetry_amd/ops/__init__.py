@@ -890,11 +890,17 @@ def residual_conv(x, w, state, cu_q, row_seq, prev_row, runs, out, save_slot=Non
         reference.conv_state_update(x, state, cu_q, prev_row, save_slot, runs)
 
 
-def post_rms_norm(x, alpha, delta, w, eps):
-    """Norm after the sum, in place on the fp32 stream: x = (alpha x + delta) / rms(alpha x + delta) * w."""
+def post_rms_norm(x, alpha, delta, w, eps, conv_w=None, conv_state=None, prev_row=None, save_slot=None, h=None):
+    """Norm after the sum, in place on the fp32 stream: x = (alpha x + delta) / rms(alpha x + delta) * w.  With ``h`` (steps
+    whose rows are runs of their own: decode) the same launch makes the next sublayer's input h = x + conv(x) as
+    ``residual_conv`` does, from the row's carried taps in ``conv_state``, and moves them on."""
     if _gpu(x):
-        return _hyb().post_rms_norm(x, float(alpha), delta, w, float(eps))
-    return reference.post_rms_norm(x, alpha, delta, w, eps)
+        return _hyb().post_rms_norm(x, float(alpha), delta, w, float(eps), conv_w, conv_state, prev_row, save_slot, h)
+    reference.post_rms_norm(x, alpha, delta, w, eps)
+    if h is not None:
+        runs = x.shape[0]
+        reference.residual_conv(x, conv_w, conv_state, None, prev_row, runs, h)
+        reference.conv_state_update(x, conv_state, None, prev_row, save_slot, runs)
 
 
 def qk_norm_cache(z, H, G, dk, dv, wq, wk, q_mult, eps, slots, q_out, k_cache, v_cache):

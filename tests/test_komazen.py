@@ -178,8 +178,8 @@ def test_layer_by_layer_against_the_oracle(tmp_path):
     seen = []
     real = ops.post_rms_norm
 
-    def spy(x, alpha, delta, w, eps):
-        real(x, alpha, delta, w, eps)
+    def spy(x, *a):
+        real(x, *a)
         seen.append(x.clone())
 
     ops.post_rms_norm = spy
@@ -416,6 +416,34 @@ def test_input_convolution_with_carried_taps(device, taps):
     got_a.append(o)
     assert float((torch.cat(got_a) - want_a).abs().max()) < 1e-5
     assert float((torch.cat(got_b) - want_b).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("taps,d", [(1, 24), (3, 40), (4, 2500)])
+def test_norm_and_convolution_in_one_launch(device, taps, d):
+    """Decode rows: post_rms_norm with the convolution's arguments equals the norm followed by residual_conv and the
+    state update; a row at position 0 reads no state, a row without a slot writes none."""
+    say("op post_rms_norm + conv", device, taps, d)
+    torch.manual_seed(taps)
+    T = 5
+    x0, delta, w, cw = torch.randn(T, d), torch.randn(T, d), torch.rand(d) + 0.5, torch.randn(d, taps) * 0.4
+    st0 = torch.randn(7, taps - 1, d)
+    prev = torch.tensor([-2, -1, -(4 + 2), -(6 + 2), -1], dtype=torch.int32)     # slots 0, -, 4, 6, - (padding row)
+    save = torch.tensor([0, 3, 4, 6, -1], dtype=torch.int32)
+    xa, xb, delta, w, cw, sa, sb, prev, save = _dev(device, x0.clone(), x0.clone(), delta, w, cw, st0.clone(), st0.clone(),
+                                                    prev, save)
+    ha, hb = torch.empty(T, d, device=device), torch.empty(T, d, device=device)
+    ops.post_rms_norm(xa, 2.25, delta, w, 1e-5)
+    ops.residual_conv(xa, cw, sa, None, None, prev, T, ha)
+    ops.conv_state_update(xa, sa, None, prev, save, T)
+    ops.post_rms_norm(xb, 2.25, delta, w, 1e-5, cw, sb, prev, save, hb)
+    assert torch.allclose(xa, xb, atol=1e-6) and torch.allclose(ha, hb, atol=1e-5) and torch.allclose(sa, sb, atol=1e-6)
+    want = O.rms_norm(2.25 * x0.double() + delta.cpu().double(), w.cpu().double(), 1e-5)
+    assert float((xb.cpu().double() - want).abs().max()) < 1e-5
+    if taps > 1:      # row 0 continued slot 0: its input one place back is that slot's newest tap
+        h0 = want[0] + cw.cpu().double()[:, -1] * want[0] + (cw.cpu().double()[:, :-1].T * st0[0].double()).sum(0)
+        assert float((hb.cpu().double()[0] - h0).abs().max()) < 1e-4
+        assert torch.equal(sb.cpu()[1], st0[1]) and torch.equal(sb.cpu()[5], st0[5])        # untouched slots
 
 
 @pytest.mark.parametrize("device", DEVICES)
