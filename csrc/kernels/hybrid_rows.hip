@@ -339,16 +339,13 @@ __global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
 }
 
 // one workgroup per row; the row's sums stay in registers between the two passes (up to PER columns per thread, wider
-// rows recompute).  With `cv` (rows that are runs of their own: decode steps) the same launch also makes the next
-// sublayer's input h = x_new + conv(x_new) from the row's carried taps and moves the taps on: a thread owns its columns
-// of the row and of the row's slot.
+// rows recompute)
 template <typename T, int BT>
 __global__ __launch_bounds__(BT) void post_rms_norm_kernel(float* __restrict__ x, float alpha, const T* __restrict__ delta,
-                                                           const float* __restrict__ w, float eps, int d, NormConvArgs cv) {
+                                                           const float* __restrict__ w, float eps, int d) {
   __shared__ float scratch[BT / 64];
   constexpr int PER = 8;
-  const int row = blockIdx.x;
-  const long long o = (long long)row * d;
+  const long long o = (long long)blockIdx.x * d;
   float v[PER];
   float sq = 0.f;
 #pragma unroll
@@ -362,39 +359,78 @@ __global__ __launch_bounds__(BT) void post_rms_norm_kernel(float* __restrict__ x
     sq += u * u;
   }
   const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
-  const float* st = nullptr;
-  float* dst = nullptr;
-  if (cv.h) {
-    const int pr = cv.prev_row[row], sv = cv.save_slot[row];
-    if (pr <= -2) st = cv.state + (long long)(-(pr + 2)) * cv.state_stride;
-    if (sv >= 0) dst = cv.state + (long long)sv * cv.state_stride;
-  }
-  auto finish = [&](int c, float xn) {
-    x[o + c] = xn;
-    if (!cv.h) return;
-    const int taps = cv.taps, keep = taps - 1;
-    const float* cw = cv.w + (long long)c * taps;
-    float old[MAX_TAPS];
-    float acc = xn + cw[keep] * xn;
-#pragma unroll
-    for (int m = 0; m < MAX_TAPS; ++m)
-      if (m < keep) {
-        old[m] = st ? st[(long long)m * d + c] : 0.f;     // old[m]: the input keep - m positions back
-        acc += cw[m] * old[m];
-      }
-    reinterpret_cast<T*>(cv.h)[o + c] = (T)acc;
-    if (dst) {
-#pragma unroll
-      for (int m = 0; m < MAX_TAPS; ++m)
-        if (m < keep) dst[(long long)m * d + c] = m + 1 < keep ? old[m + 1] : xn;
-    }
-  };
   // (each thread rewrites only the columns it read itself)
-  for (int c = threadIdx.x + PER * BT; c < d; c += BT) finish(c, (alpha * x[o + c] + (float)delta[o + c]) * r * w[c]);
+  for (int c = threadIdx.x + PER * BT; c < d; c += BT) x[o + c] = (alpha * x[o + c] + (float)delta[o + c]) * r * w[c];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int c = threadIdx.x + i * BT;
-    if (c < d) finish(c, v[i] * r * w[c]);
+    if (c < d) x[o + c] = v[i] * r * w[c];
+  }
+}
+
+// The same for rows that are runs of their own (decode steps), and in the same launch the next sublayer's input
+// h = x_new + conv(x_new) from the row's carried taps, which move on: a thread owns its columns of the row and of the
+// row's slot.  One column pass of BT threads keeps its weights, taps and carried inputs in registers, loaded before the
+// row's reduction so that only the arithmetic follows it; wider rows take further passes.  TAPS: the tap count where it
+// is at most 8 (exact register arrays), 0 for any count up to MAX_TAPS.
+template <typename T, int BT, int TAPS>
+__global__ __launch_bounds__(BT) void post_rms_norm_conv_kernel(float* __restrict__ x, float alpha,
+                                                                const T* __restrict__ delta, const float* __restrict__ w,
+                                                                float eps, int d, NormConvArgs cv) {
+  __shared__ float scratch[BT / 64];
+  constexpr int KEEP = TAPS ? TAPS - 1 : MAX_TAPS - 1;
+  const int row = blockIdx.x;
+  const long long o = (long long)row * d;
+  const int taps = TAPS ? TAPS : cv.taps, keep = taps - 1;
+  const int pr = cv.prev_row[row], sv = cv.save_slot[row];
+  const float* st = pr <= -2 ? cv.state + (long long)(-(pr + 2)) * cv.state_stride : nullptr;
+  float* dst = sv >= 0 ? cv.state + (long long)sv * cv.state_stride : nullptr;
+  const int c0 = threadIdx.x;
+  float v0 = 0.f, w0 = 0.f, cw[KEEP + 1], old[KEEP];
+  if (c0 < d) {
+    v0 = alpha * x[o + c0] + (float)delta[o + c0];
+    w0 = w[c0];
+#pragma unroll
+    for (int m = 0; m <= KEEP; ++m)
+      if (m <= keep) cw[m] = cv.w[(long long)c0 * taps + m];
+#pragma unroll
+    for (int m = 0; m < KEEP; ++m)
+      if (m < keep) old[m] = st ? st[(long long)m * d + c0] : 0.f;      // old[m]: the input keep - m positions back
+  }
+  float sq = v0 * v0;
+  for (int c = c0 + BT; c < d; c += BT) {
+    const float u = alpha * x[o + c] + (float)delta[o + c];
+    sq += u * u;
+  }
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
+  T* h = reinterpret_cast<T*>(cv.h);
+  for (int c = c0 + BT; c < d; c += BT) {     // further passes: loads after the reduction
+    const float xn = (alpha * x[o + c] + (float)delta[o + c]) * r * w[c];
+    const float* cwp = cv.w + (long long)c * taps;
+    float acc = xn + cwp[keep] * xn, prev = 0.f;
+    for (int m = 0; m < keep; ++m) {
+      const float ov = st ? st[(long long)m * d + c] : 0.f;
+      acc += cwp[m] * ov;
+      if (dst && m > 0) dst[(long long)(m - 1) * d + c] = ov;   // (this thread alone reads and writes column c of the slot)
+      prev = ov;
+    }
+    (void)prev;
+    if (dst && keep > 0) dst[(long long)(keep - 1) * d + c] = xn;
+    x[o + c] = xn;
+    h[o + c] = (T)acc;
+  }
+  if (c0 >= d) return;
+  const float xn = v0 * r * w0;
+  float acc = xn + cw[keep] * xn;
+#pragma unroll
+  for (int m = 0; m < KEEP; ++m)
+    if (m < keep) acc += cw[m] * old[m];
+  x[o + c0] = xn;
+  h[o + c0] = (T)acc;
+  if (dst) {
+#pragma unroll
+    for (int m = 0; m < KEEP; ++m)
+      if (m < keep) dst[(long long)m * d + c0] = m + 1 < keep ? old[m + 1 < KEEP ? m + 1 : m] : xn;
   }
 }
 
@@ -583,13 +619,32 @@ void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s) {
   DISPATCH_T(f32, residual_conv_kernel<T><<<grid, NT, 0, s>>>(a);)
 }
 
+template <typename T, int BT>
+static void post_rms_norm_conv_taps(float* x, float alpha, const void* delta, const float* w, float eps, int T_, int d,
+                                    const NormConvArgs& cv, hipStream_t s) {
+  switch (cv.taps) {
+    case 2: post_rms_norm_conv_kernel<T, BT, 2><<<T_, BT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv); break;
+    case 3: post_rms_norm_conv_kernel<T, BT, 3><<<T_, BT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv); break;
+    case 4: post_rms_norm_conv_kernel<T, BT, 4><<<T_, BT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv); break;
+    default: post_rms_norm_conv_kernel<T, BT, 0><<<T_, BT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv); break;
+  }
+}
+
 void launch_post_rms_norm(float* x, float alpha, const void* delta, const float* w, float eps, int T_, int d,
                           const NormConvArgs& cv, int f32, hipStream_t s) {
   if (T_ <= 0) return;
+  if (cv.h) {
+    if (d > 256) {
+      DISPATCH_T(f32, (post_rms_norm_conv_taps<T, 1024>(x, alpha, delta, w, eps, T_, d, cv, s));)
+    } else {
+      DISPATCH_T(f32, (post_rms_norm_conv_taps<T, NT>(x, alpha, delta, w, eps, T_, d, cv, s));)
+    }
+    return;
+  }
   if (wide_rows(T_, d)) {
-    DISPATCH_T(f32, (post_rms_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv));)
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
   } else {
-    DISPATCH_T(f32, (post_rms_norm_kernel<T, NT><<<T_, NT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d, cv));)
+    DISPATCH_T(f32, (post_rms_norm_kernel<T, NT><<<T_, NT, 0, s>>>(x, alpha, (const T*)delta, w, eps, d));)
   }
 }
 

@@ -17,6 +17,26 @@ namespace {
 
 constexpr int MAX_VCOLS = 8;  // value columns per lane: dv <= 512
 
+// Value columns of a lane.  Plain: lane + 64 i.  PAIR (even dv): two neighbouring columns per load, 128 (i / 2) + 2 lane
+// + (i & 1): half the load instructions of the value walk, which is a chain of dependent batches in a decode step.
+template <bool PAIR>
+SYM_DEV int vcol(int lane, int i) {
+  return PAIR ? 128 * (i >> 1) + 2 * lane + (i & 1) : lane + 64 * i;
+}
+template <bool PAIR>
+SYM_DEV int vcols(int dv) {   // accumulator slots in use
+  return PAIR ? 2 * ((dv + 127) >> 7) : (dv + 63) >> 6;
+}
+SYM_DEV void load_pair(const bf16* p, float& a, float& b) {
+  const unsigned int w = *reinterpret_cast<const unsigned int*>(p);
+  a = __uint_as_float(w << 16);
+  b = __uint_as_float(w & 0xffff0000u);
+}
+SYM_DEV void load_pair(const float* p, float& a, float& b) {
+  const float2 w = *reinterpret_cast<const float2*>(p);
+  a = w.x, b = w.y;
+}
+
 // cache row of position kp of a sequence (block table bt): a shift and a mask for power-of-two blocks
 SYM_DEV long long cache_row(const int* __restrict__ bt, int kp, int BS, int shift) {
   return shift >= 0 ? ((long long)bt[kp >> shift] << shift) + (kp & (BS - 1)) : (long long)bt[kp / BS] * BS + kp % BS;
@@ -63,14 +83,14 @@ SYM_DEV void dot_rows(const T* __restrict__ k, const float* __restrict__ qs, int
 // once for the REP accumulators.  Wave w walks the key tiles w, w + NW, ... of the row's window with its own running
 // max / sum / accumulators; the waves' partial results meet in LDS at the end (rows of a decode step have few (row,
 // head) pairs and long windows: NW > 1 shortens each wave's walk).  Dynamic LDS: REP dk + NW REP (2 + 64 nvc) floats.
-template <typename T, int NW, int REP>
+template <typename T, int NW, int REP, bool PAIR>
 __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArgs a) {
   extern __shared__ float lds[];
   float* qs = lds;                      // [REP][dk]
   float* part = lds + REP * a.dk;       // [NW][REP][2 + 64 nvc]: m, l, acc
   const int h0 = blockIdx.x * REP, row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = h0 / (a.H / a.G);
-  const int nvc = (a.dv + 63) >> 6, pstride = 2 + 64 * nvc;
+  const int nvc = vcols<PAIR>(a.dv), pstride = 2 + 64 * nvc;
   const int p = a.positions[row];
   const int j0 = max(0, p - a.window + 1);
   const int* bt = a.block_tables + (long long)a.row_seq[row] * a.max_blocks;
@@ -117,7 +137,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     const int vslot = (int)slot;              // (cache rows fit 31 bits: checked by the op layer)
     // value rows VB at a time: their cache rows come lane by lane from the scoring phase (no block-table walk in this
     // loop), the loads of a batch are issued together and serve all REP heads
-    constexpr int VB = REP >= 4 ? 4 : 8;
+    constexpr int VB = REP >= 4 ? 4 : (PAIR ? 16 : 8);
     for (int jj = 0; jj < nt; jj += VB) {
       float pw[REP][VB];
       const T* vr[VB];
@@ -127,17 +147,36 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
 #pragma unroll
         for (int r = 0; r < REP; ++r) pw[r][u] = __shfl(w[r], jj + u, 64);
       }
+      if constexpr (PAIR) {
 #pragma unroll
-      for (int i = 0; i < MAX_VCOLS; ++i) {
-        const int c = lane + 64 * i;
-        if (c < a.dv) {
-          float vv[VB];
+        for (int i = 0; i < MAX_VCOLS; i += 2) {
+          const int c = vcol<true>(lane, i);
+          if (c < a.dv) {
+            float v0[VB], v1[VB];
 #pragma unroll
-          for (int u = 0; u < VB; ++u) vv[u] = (float)vr[u][c];
+            for (int u = 0; u < VB; ++u) load_pair(vr[u] + c, v0[u], v1[u]);
 #pragma unroll
-          for (int r = 0; r < REP; ++r)
+            for (int r = 0; r < REP; ++r)
 #pragma unroll
-            for (int u = 0; u < VB; ++u) acc[r][i] += pw[r][u] * vv[u];
+              for (int u = 0; u < VB; ++u) {
+                acc[r][i] += pw[r][u] * v0[u];
+                acc[r][i + 1] += pw[r][u] * v1[u];
+              }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < MAX_VCOLS; ++i) {
+          const int c = lane + 64 * i;
+          if (c < a.dv) {
+            float vv[VB];
+#pragma unroll
+            for (int u = 0; u < VB; ++u) vv[u] = (float)vr[u][c];
+#pragma unroll
+            for (int r = 0; r < REP; ++r)
+#pragma unroll
+              for (int u = 0; u < VB; ++u) acc[r][i] += pw[r][u] * vv[u];
+          }
         }
       }
     }
@@ -183,18 +222,18 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     T* o = reinterpret_cast<T*>(a.out) + ((long long)row * a.H + h) * a.dv;
 #pragma unroll
     for (int i = 0; i < MAX_VCOLS; ++i) {
-      const int c = lane + 64 * i;
-      if (c < a.dv) o[c] = (T)(acc[r][i] * inv);
+      const int c = vcol<PAIR>(lane, i);
+      if (i < nvc && c < a.dv) o[c] = (T)(acc[r][i] * inv);
     }
   }
 }
 
-template <typename T, int NW, int REP>
+template <typename T, int NW, int REP, bool PAIR>
 void launch_wave_rep(const WindowAttnArgs& a, hipStream_t s) {
   dim3 grid(a.H / REP, a.T);
-  const int nvc = (a.dv + 63) / 64;
+  const int nvc = PAIR ? 2 * ((a.dv + 127) / 128) : (a.dv + 63) / 64;
   const size_t lds = (size_t)(REP * a.dk + (NW > 1 ? NW * REP * (2 + 64 * nvc) : 0)) * sizeof(float);
-  window_attn_wave_kernel<T, NW, REP><<<grid, 64 * NW, lds, s>>>(a);
+  window_attn_wave_kernel<T, NW, REP, PAIR><<<grid, 64 * NW, lds, s>>>(a);
 }
 
 template <typename T, int NW>
@@ -205,10 +244,14 @@ void launch_wave(const WindowAttnArgs& a, hipStream_t s) {
   const int rep = a.H / a.G, nvc = (a.dv + 63) / 64;
   const bool fits = (size_t)(rep * a.dk + NW * rep * (2 + 64 * nvc)) * sizeof(float) <= 60 * 1024 && rep * nvc <= 16 &&
                     (long long)a.T * a.G * NW >= 1024;
-  if (rep == 8 && fits) launch_wave_rep<T, NW, 8>(a, s);
-  else if (rep == 4 && fits) launch_wave_rep<T, NW, 4>(a, s);
-  else if (rep == 2 && fits) launch_wave_rep<T, NW, 2>(a, s);
-  else launch_wave_rep<T, NW, 1>(a, s);
+  if constexpr (NW <= 8) {
+    if (rep == 8 && fits) return launch_wave_rep<T, NW, 8, false>(a, s);
+    if (rep == 4 && fits) return launch_wave_rep<T, NW, 4, false>(a, s);
+    if (rep == 2 && fits) return launch_wave_rep<T, NW, 2, false>(a, s);
+  }
+  // one head per workgroup: value rows two columns per load where the head size is even (rows stay 4-byte aligned)
+  if (a.dv % 2 == 0) launch_wave_rep<T, NW, 1, true>(a, s);
+  else launch_wave_rep<T, NW, 1, false>(a, s);
 }
 
 // ---- tiled kernel for prompt rows (bf16, head sizes DK = DV in {32, 64, 96, 128}) --------------------------------
@@ -423,16 +466,21 @@ int launch_window_attn(const WindowAttnArgs& args, int f32, int impl, hipStream_
     }
   }
   // few (row, head) pairs and a long window (decode steps): several waves per pair
+  // (a handful of rows over a thousand keys or more: sixteen waves, one or two key tiles each)
   const long long pairs = (long long)a.T * a.H;
-  const int nw = pairs >= 8192 || a.window <= 128 ? 1 : (a.window <= 512 || pairs >= 2048 ? 4 : 8);
+  const long long reach = min((long long)a.window, (long long)a.max_blocks * a.BS);   // keys a row can see at most
+  const int nw = pairs >= 8192 || a.window <= 128 ? 1
+                 : (a.window <= 512 || pairs >= 2048 ? 4 : (pairs <= 512 && reach >= 1024 ? 16 : 8));
   if (f32) {
     if (nw == 1) launch_wave<float, 1>(a, s);
     else if (nw == 4) launch_wave<float, 4>(a, s);
-    else launch_wave<float, 8>(a, s);
+    else if (nw == 8) launch_wave<float, 8>(a, s);
+    else launch_wave<float, 16>(a, s);
   } else {
     if (nw == 1) launch_wave<bf16, 1>(a, s);
     else if (nw == 4) launch_wave<bf16, 4>(a, s);
-    else launch_wave<bf16, 8>(a, s);
+    else if (nw == 8) launch_wave<bf16, 8>(a, s);
+    else launch_wave<bf16, 16>(a, s);
   }
   return 0;
 }
