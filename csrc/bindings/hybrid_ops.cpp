@@ -472,7 +472,10 @@ void residual_conv(const Tensor& x, const Tensor& w, Tensor& state, const OptTen
   dtype(x, at::kFloat, "x");
   dtype(w, at::kFloat, "w");
   dtype(state, at::kFloat, "state");
-  ConvArgs a = conv_args(x, w, std::nullopt, state, cu_q, row_seq, prev_row, save_slot, runs, 1);
+  // (the taps are tap-major here, [taps, C]: conv_args checks the channel-major form of causal_conv_silu)
+  ConvArgs a = conv_args(x, std::nullopt, std::nullopt, state, cu_q, row_seq, prev_row, save_slot, runs, 1);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == a.taps && w.size(1) == a.C, "residual_conv: w [taps, C]");
+  a.w = w.data_ptr();
   TORCH_CHECK(!cu_q.has_value() || row_seq.has_value(), "residual_conv: cu_q without row_seq");
   TORCH_CHECK(!(cu_q.has_value() && save_slot.has_value()), "residual_conv: the taps move on in this launch only where "
               "every row is a run of its own");
@@ -497,8 +500,8 @@ void post_rms_norm(Tensor& x, double alpha, const Tensor& delta, const Tensor& w
     dtype(*conv_state, at::kFloat, "conv_state");
     dtype(*prev_row, at::kInt, "prev_row");
     dtype(*save_slot, at::kInt, "save_slot");
-    TORCH_CHECK(conv_w->dim() == 2 && conv_w->size(0) == d && conv_state->dim() == 3 && conv_state->size(2) == d &&
-                    conv_state->size(1) + 1 == conv_w->size(1) && conv_w->size(1) <= 16 && h->numel() == T * d &&
+    TORCH_CHECK(conv_w->dim() == 2 && conv_w->size(1) == d && conv_state->dim() == 3 && conv_state->size(2) == d &&
+                    conv_state->size(1) + 1 == conv_w->size(0) && conv_w->size(0) <= 16 && h->numel() == T * d &&
                     prev_row->numel() >= T && save_slot->numel() >= T, "post_rms_norm: convolution shapes");
     cv.w = ptr<float>(*conv_w);
     cv.state = ptr<float>(*conv_state);
@@ -506,7 +509,7 @@ void post_rms_norm(Tensor& x, double alpha, const Tensor& delta, const Tensor& w
     cv.prev_row = ptr<int>(*prev_row);
     cv.save_slot = ptr<int>(*save_slot);
     cv.h = h->data_ptr();
-    cv.taps = (int)conv_w->size(1);
+    cv.taps = (int)conv_w->size(0);
   }
   launch_post_rms_norm(ptr<float>(x), (float)alpha, delta.data_ptr(), ptr<float>(w), (float)eps, (int)T, (int)d, cv, f32,
                        cur_stream(x));

@@ -80,14 +80,15 @@ void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* 
 // x[row] = table[token] * scale, token as for launch_embed_norm
 void launch_embed_scale(const int* ids, const int* src, const int* prev, const void* table, float scale, float* x, int T,
                         int d, int f32, hipStream_t s);
-// ConvArgs with xin / state / w fp32 and no bias: out (activation dtype) = x + sum_j w[c][taps - 1 - j] x[t - j][c];
+// ConvArgs with xin / state / w fp32, w tap-major [taps][C], no bias: out (activation dtype) = x + sum_j w[taps - 1 - j][c]
+// x[t - j][c];
 // the carried taps are then stored by launch_conv_state_update(a, 1, s) -- or by this launch itself where every row is a
 // run of its own (cu_q null) and save_slot is given
 void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s);
 // x = (alpha x + delta) / rms * w, in place on the fp32 stream (delta in the activation dtype).  With cv.h set (every row
 // a run of its own): also h = x_new + conv(x_new) over the row's carried taps (as launch_residual_conv), which move on
 struct NormConvArgs {
-  const float* w;        // [d][taps]
+  const float* w;        // [taps][d]
   float* state;          // [slots][taps - 1][d]
   long long state_stride;
   const int* prev_row;

@@ -32,6 +32,11 @@ SYM_DEV float ldf(const void* p, int f32, long long i) {
 
 SYM_DEV float sigmoidf(float v) { return 1.f / (1.f + expf(-v)); }
 SYM_DEV float silu_exact(float v) { return v / (1.f + expf(-v)); }
+// 0.5 v (1 + tanh(u)) = v sigmoid(2 u), u = sqrt(2 / pi) (v + 0.044715 v^3)
+SYM_DEV float gelu_tanh_exact(float v) {
+  const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  return v / (1.f + expf(-2.f * u));
+}
 
 template <typename T, int BT>
 __global__ __launch_bounds__(BT) void embed_norm_kernel(const int* __restrict__ ids, const int* __restrict__ src,
@@ -312,13 +317,13 @@ __global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
   const int pr = a.prev_row[s0];
   const float* st = pr <= -2 ? reinterpret_cast<const float*>(a.state) + (long long)(-(pr + 2)) * a.state_stride : nullptr;
   const float* x = reinterpret_cast<const float*>(a.xin);
-  const float* w = reinterpret_cast<const float*>(a.w) + (long long)c * taps;
+  const float* w = reinterpret_cast<const float*>(a.w) + c;     // [taps][C]
   float acc = x[(long long)row * a.ldx + c];
   for (int i = 0; i < taps; ++i) {       // i positions back
     float v = 0.f;
     if (i <= j) v = x[(long long)(row - i) * a.ldx + c];
     else if (st) v = st[(long long)(taps - 1 - (i - j)) * a.C + c];
-    acc += w[taps - 1 - i] * v;
+    acc += w[(long long)(taps - 1 - i) * a.C] * v;
   }
   reinterpret_cast<T*>(a.out)[(long long)row * a.C + c] = (T)acc;
   // rows that are runs of their own (decode steps): this thread alone reads and writes its channel of the row's slot, so
@@ -335,6 +340,56 @@ __global__ __launch_bounds__(NT) void residual_conv_kernel(ConvArgs a) {
 #pragma unroll
     for (int m = 0; m < MAX_TAPS; ++m)
       if (m < keep) dst[(long long)m * a.C + c] = vals[m];
+  }
+}
+
+// The same for prompt-sized launches with C and the row stride multiples of 4: a thread takes four channels (16-byte
+// loads of the stream and of the tap-major weights, which it keeps in registers) and walks CONV_ROWS consecutive rows,
+// grid (ceil(T / CONV_ROWS), ceil(C / 4 / NT)).  The taps never move on here (runs of several rows).
+constexpr int CONV_ROWS = 8;
+template <typename T, int TAPS>     // TAPS: the tap count where it is at most 4, else 0 (any count up to MAX_TAPS)
+__global__ __launch_bounds__(NT) void residual_conv_vec_kernel(ConvArgs a) {
+  constexpr int NTAP = TAPS ? TAPS : MAX_TAPS;
+  const int row0 = blockIdx.x * CONV_ROWS, c = (blockIdx.y * NT + threadIdx.x) * 4;
+  if (c >= a.C) return;
+  const int taps = TAPS ? TAPS : a.taps;
+  const float* x = reinterpret_cast<const float*>(a.xin);
+  float4 wv[NTAP];     // wv[i]: the weights of the input i positions back
+#pragma unroll
+  for (int i = 0; i < NTAP; ++i)
+    if (i < taps)
+      wv[i] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.w) + (long long)(taps - 1 - i) * a.C + c);
+  for (int r = 0; r < CONV_ROWS; ++r) {
+    const int row = row0 + r;
+    if (row >= a.T) return;
+    const int s0 = a.cu_q ? a.cu_q[a.row_seq[row]] : row;
+    const int j = row - s0;
+    const float* st = nullptr;
+    if (j < taps - 1) {
+      const int pr = a.prev_row[s0];
+      if (pr <= -2) st = reinterpret_cast<const float*>(a.state) + (long long)(-(pr + 2)) * a.state_stride;
+    }
+    const float4 own = *reinterpret_cast<const float4*>(x + (long long)row * a.ldx + c);
+    float4 acc = own;
+#pragma unroll
+    for (int i = 0; i < NTAP; ++i) {       // i positions back
+      if (i < taps) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i == 0) v = own;
+        else if (i <= j) v = *reinterpret_cast<const float4*>(x + (long long)(row - i) * a.ldx + c);
+        else if (st) v = *reinterpret_cast<const float4*>(st + (long long)(taps - 1 - (i - j)) * a.C + c);
+        const float4 wt = wv[i];
+        acc.x += wt.x * v.x, acc.y += wt.y * v.y, acc.z += wt.z * v.z, acc.w += wt.w * v.w;
+      }
+    }
+    T* o = reinterpret_cast<T*>(a.out) + (long long)row * a.C + c;
+    if constexpr (sizeof(T) == 2) {
+      bf16x4 pk;
+      pk[0] = (bf16)acc.x, pk[1] = (bf16)acc.y, pk[2] = (bf16)acc.z, pk[3] = (bf16)acc.w;
+      *reinterpret_cast<bf16x4*>(o) = pk;
+    } else {
+      *reinterpret_cast<float4*>(o) = acc;
+    }
   }
 }
 
@@ -392,7 +447,7 @@ __global__ __launch_bounds__(BT) void post_rms_norm_conv_kernel(float* __restric
     w0 = w[c0];
 #pragma unroll
     for (int m = 0; m <= KEEP; ++m)
-      if (m <= keep) cw[m] = cv.w[(long long)c0 * taps + m];
+      if (m <= keep) cw[m] = cv.w[(long long)m * d + c0];
 #pragma unroll
     for (int m = 0; m < KEEP; ++m)
       if (m < keep) old[m] = st ? st[(long long)m * d + c0] : 0.f;      // old[m]: the input keep - m positions back
@@ -406,11 +461,11 @@ __global__ __launch_bounds__(BT) void post_rms_norm_conv_kernel(float* __restric
   T* h = reinterpret_cast<T*>(cv.h);
   for (int c = c0 + BT; c < d; c += BT) {     // further passes: loads after the reduction
     const float xn = (alpha * x[o + c] + (float)delta[o + c]) * r * w[c];
-    const float* cwp = cv.w + (long long)c * taps;
-    float acc = xn + cwp[keep] * xn, prev = 0.f;
+    const float* cwp = cv.w + c;      // [taps][d]
+    float acc = xn + cwp[(long long)keep * d] * xn, prev = 0.f;
     for (int m = 0; m < keep; ++m) {
       const float ov = st ? st[(long long)m * d + c] : 0.f;
-      acc += cwp[m] * ov;
+      acc += cwp[(long long)m * d] * ov;
       if (dst && m > 0) dst[(long long)(m - 1) * d + c] = ov;   // (this thread alone reads and writes column c of the slot)
       prev = ov;
     }
@@ -476,9 +531,26 @@ __global__ __launch_bounds__(NT) void gelu_tanh_mul_kernel(const T* __restrict__
   for (long long i = (long long)blockIdx.x * NT + threadIdx.x; i < n; i += (long long)gridDim.x * NT) {
     const long long r = i / F, c = i - r * F;
     const float gv = (float)g[r * ldg + c];
-    const float t = tanhf(0.7978845608028654f * (gv + 0.044715f * gv * gv * gv));
-    out[i] = (T)(0.5f * gv * (1.f + t) * (float)u[r * ldu + c]);
+    out[i] = (T)(gelu_tanh_exact(gv) * (float)u[r * ldu + c]);
   }
+}
+
+// bf16, F and both row strides multiples of 8, 16-byte aligned views: eight columns per thread (prompt-sized launches
+// are bandwidth-bound)
+__global__ __launch_bounds__(NT) void gelu_tanh_mul_vec_kernel(const bf16* __restrict__ g, long long ldg,
+                                                               const bf16* __restrict__ u, long long ldu,
+                                                               bf16* __restrict__ out, long long nvec, int F) {
+  const long long i = (long long)blockIdx.x * NT + threadIdx.x;
+  if (i >= nvec) return;
+  const int fv = F >> 3;
+  const long long r = i / fv;
+  const int c = (int)(i - r * fv) * 8;
+  float gv[8], uv[8], y[8];
+  load8(g + r * ldg + c, gv);
+  load8(u + r * ldu + c, uv);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = gelu_tanh_exact(gv[j]) * uv[j];
+  store8(out + r * F + c, y);
 }
 
 template <typename T>
@@ -615,6 +687,22 @@ void launch_embed_scale(const int* ids, const int* src, const int* prev, const v
 
 void launch_residual_conv(const ConvArgs& a, int f32, hipStream_t s) {
   if (a.T <= 0) return;
+  const bool moves = !a.cu_q && a.save_slot;      // the launch that also moves the taps on keeps one channel per thread
+  if (!moves && a.T >= 256 && a.C % 4 == 0 && a.ldx % 4 == 0 && (reinterpret_cast<uintptr_t>(a.xin) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(a.state) & 15) == 0 && a.state_stride % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(a.w) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0) {
+    dim3 grid((a.T + CONV_ROWS - 1) / CONV_ROWS, (a.C / 4 + NT - 1) / NT);
+    if (a.taps == 4) {
+      DISPATCH_T(f32, (residual_conv_vec_kernel<T, 4><<<grid, NT, 0, s>>>(a));)
+    } else if (a.taps == 3) {
+      DISPATCH_T(f32, (residual_conv_vec_kernel<T, 3><<<grid, NT, 0, s>>>(a));)
+    } else if (a.taps == 2) {
+      DISPATCH_T(f32, (residual_conv_vec_kernel<T, 2><<<grid, NT, 0, s>>>(a));)
+    } else {
+      DISPATCH_T(f32, (residual_conv_vec_kernel<T, 0><<<grid, NT, 0, s>>>(a));)
+    }
+    return;
+  }
   dim3 grid(a.T, (a.C + NT - 1) / NT);
   DISPATCH_T(f32, residual_conv_kernel<T><<<grid, NT, 0, s>>>(a);)
 }
@@ -657,6 +745,13 @@ void launch_qk_norm_cache(const QkNormArgs& a, int T_, int f32, hipStream_t s) {
 void launch_gelu_tanh_mul(const void* gate, long long ldg, const void* up, long long ldu, void* out, int R, int F, int f32,
                           hipStream_t s) {
   if (R <= 0) return;
+  const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (!f32 && F % 8 == 0 && ldg % 8 == 0 && ldu % 8 == 0 && al(gate) && al(up) && al(out)) {
+    const long long nvec = (long long)R * F / 8;
+    gelu_tanh_mul_vec_kernel<<<(unsigned)((nvec + NT - 1) / NT), NT, 0, s>>>((const bf16*)gate, ldg, (const bf16*)up, ldu,
+                                                                           (bf16*)out, nvec, F);
+    return;
+  }
   DISPATCH_T(f32, gelu_tanh_mul_kernel<T><<<ew_grid((long long)R * F), NT, 0, s>>>((const T*)gate, ldg, (const T*)up,
                                                                                    ldu, (T*)out, R, F);)
 }

@@ -144,7 +144,10 @@ class KomazenLM:
         def f(name):
             return w[p + name].float().contiguous()
 
-        P = {"kind": layer.type, "mixer": m, "mlp": layer.mlp, "norm1": f("norm1"), "canon1": f("canon1"), "o": t("mix.o")}
+        def taps(name):      # [width, taps] in the checkpoint -> tap-major, so that neighbouring channels load together
+            return w[p + name].float().t().contiguous()
+
+        P = {"kind": layer.type, "mixer": m, "mlp": layer.mlp, "norm1": f("norm1"), "canon1": taps("canon1"), "o": t("mix.o")}
         if layer.type == "latent_attention":
             if m.kv_rank > 512:
                 raise NotImplementedError(f"layer {i}: kv_rank {m.kv_rank} > 512 (latent_attn's accumulator registers)")
@@ -166,7 +169,7 @@ class KomazenLM:
             P["temp"] = f("mix.temp")
             P["bias"] = torch.stack([f("mix.r1"), f("mix.r2")]).contiguous()           # [2, H]
         if layer.mlp is not None:
-            P["norm2"], P["canon2"] = f("norm2"), f("canon2")
+            P["norm2"], P["canon2"] = f("norm2"), taps("canon2")
             P["w_gu"] = torch.cat([t("mlp.gate"), t("mlp.up")], 0).contiguous()
             P["w_down"] = t("mlp.down")
         return P

@@ -876,8 +876,9 @@ def embed_scale(ids, table, scale, x, src=None, prev=None):
 
 
 def residual_conv(x, w, state, cu_q, row_seq, prev_row, runs, out, save_slot=None):
-    """out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j) per channel over every run of rows of the fp32 stream x (the
-    sublayer input in the activation dtype); inputs before the run come from state[slot] [taps - 1, C] fp32
+    """out_t = x_t + sum_j w[j] x_(t - taps + 1 + j) per channel (w tap-major, [taps, C] fp32) over every run of rows of
+    the fp32 stream x (the sublayer input in the activation dtype); inputs before the run come from state[slot]
+    [taps - 1, C] fp32
     (prev_row[first] <= -2) or are zero.  ``conv_state_update(x, state, ...)`` then stores the run's newest inputs; where
     every row is a run of its own (cu_q None: decode steps), ``save_slot`` makes this launch store them itself."""
     if save_slot is not None and cu_q is not None:

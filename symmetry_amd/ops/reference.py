@@ -924,8 +924,8 @@ def embed_scale(ids, table, scale, x) -> None:
 
 def residual_conv(x, w, state, cu_q, prev_row, runs, out) -> None:
     T, C = out.shape
-    taps = w.shape[1]
-    wf = w.float()
+    taps = w.shape[0]                      # w [taps, C]
+    wf = w.float().t()
     for s0, s1 in _runs(T, cu_q, runs):
         if s1 <= s0:
             continue

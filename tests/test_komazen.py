@@ -373,7 +373,7 @@ def test_input_convolution_with_carried_taps(device, taps):
     xa, xb, w = torch.randn(n, d), torch.randn(11, d), torch.randn(d, taps) * 0.5
     want_a, want_b = O.input_conv(xa.double(), w.double()), O.input_conv(xb.double(), w.double())
     state = torch.full((3, taps - 1, d), 1e4)
-    state, wd = _dev(device, state, w)
+    state, wd = _dev(device, state, w.t().contiguous())      # the op takes the taps tap-major
     i32 = torch.int32
 
     def step(rows_a, rows_b, first_a, first_b, decode=False):
@@ -419,6 +419,39 @@ def test_input_convolution_with_carried_taps(device, taps):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_prompt_sized_convolution_and_activation(device):
+    """Launches of hundreds of rows (several channels / columns per thread on the GPU): two runs, one of which continues
+    its slot; the gated activation in bfloat16 on views of a wider matrix."""
+    say("op prompt-sized rows", device)
+    torch.manual_seed(5)
+    d, taps = 72, 4
+    xa, xb, w = torch.randn(330, d), torch.randn(150, d), torch.randn(d, taps) * 0.5
+    want_a, want_b = O.input_conv(xa.double(), w.double()), O.input_conv(xb.double(), w.double())
+    state = torch.full((2, taps - 1, d), 1e4)
+    state[1] = xa[27:30]                                  # sequence a's rows 0..29 ran in an earlier step
+    x = torch.cat([xb, xa[30:]])
+    i32 = torch.int32
+    prev = torch.tensor([-1] + list(range(0, 149)) + [-(1 + 2)] + list(range(150, 449)), dtype=i32)
+    save = torch.full((450,), -1, dtype=i32)
+    save[149], save[449] = 0, 1
+    rs = torch.tensor([0] * 150 + [1] * 300, dtype=i32)
+    cu = torch.tensor([0, 150, 450], dtype=i32)
+    out = torch.empty(450, d)
+    x, w, state, prev, save, rs, cu, out = _dev(device, x, w.t().contiguous(), state, prev, save, rs, cu, out)
+    ops.residual_conv(x, w, state, cu, rs, prev, 2, out)
+    ops.conv_state_update(x, state, cu, prev, save, 2)
+    assert float((out.cpu().double()[:150] - want_b).abs().max()) < 1e-5
+    assert float((out.cpu().double()[150:] - want_a[30:]).abs().max()) < 1e-5
+    assert torch.equal(state.cpu()[0], xb[-3:]) and torch.equal(state.cpu()[1], xa[-3:])
+    gu = (torch.randn(300, 144) * 3).bfloat16()
+    act = torch.empty(300, 64, dtype=torch.bfloat16)
+    gu, act = _dev(device, gu, act)
+    ops.gelu_tanh_mul(gu[:, :64], gu[:, 72:136], act)
+    want = O.gelu_tanh(gu.cpu().double()[:, :64]) * gu.cpu().double()[:, 72:136]
+    assert float((act.cpu().double() - want).abs().max()) < 0.01 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("taps,d", [(1, 24), (3, 40), (4, 2500)])
 def test_norm_and_convolution_in_one_launch(device, taps, d):
     """Decode rows: post_rms_norm with the convolution's arguments equals the norm followed by residual_conv and the
@@ -430,8 +463,8 @@ def test_norm_and_convolution_in_one_launch(device, taps, d):
     st0 = torch.randn(7, taps - 1, d)
     prev = torch.tensor([-2, -1, -(4 + 2), -(6 + 2), -1], dtype=torch.int32)     # slots 0, -, 4, 6, - (padding row)
     save = torch.tensor([0, 3, 4, 6, -1], dtype=torch.int32)
-    xa, xb, delta, w, cw, sa, sb, prev, save = _dev(device, x0.clone(), x0.clone(), delta, w, cw, st0.clone(), st0.clone(),
-                                                    prev, save)
+    xa, xb, delta, w, cw, sa, sb, prev, save = _dev(device, x0.clone(), x0.clone(), delta, w, cw.t().contiguous(),
+                                                    st0.clone(), st0.clone(), prev, save)
     ha, hb = torch.empty(T, d, device=device), torch.empty(T, d, device=device)
     ops.post_rms_norm(xa, 2.25, delta, w, 1e-5)
     ops.residual_conv(xa, cw, sa, None, None, prev, T, ha)
@@ -441,7 +474,7 @@ def test_norm_and_convolution_in_one_launch(device, taps, d):
     want = O.rms_norm(2.25 * x0.double() + delta.cpu().double(), w.cpu().double(), 1e-5)
     assert float((xb.cpu().double() - want).abs().max()) < 1e-5
     if taps > 1:      # row 0 continued slot 0: its input one place back is that slot's newest tap
-        h0 = want[0] + cw.cpu().double()[:, -1] * want[0] + (cw.cpu().double()[:, :-1].T * st0[0].double()).sum(0)
+        h0 = want[0] + cw.cpu().double()[-1] * want[0] + (cw.cpu().double()[:-1] * st0[0].double()).sum(0)
         assert float((hb.cpu().double()[0] - h0).abs().max()) < 1e-4
         assert torch.equal(sb.cpu()[1], st0[1]) and torch.equal(sb.cpu()[5], st0[5])        # untouched slots
 
