@@ -320,6 +320,36 @@ def test_config_reader_rejects_unknown_keys_and_roundtrips(tmp_path):
     assert C.resolve("tiny-komazen").family == "komazen"
 
 
+def test_registered_model_by_name_and_checkpoint_tensors(tmp_path):
+    """The registry name runs with random weights as every other modelName does (the command line's path), and equals the
+    oracle; a checkpoint may carry the second norm / convolution of a layer without feed-forward, and no other extra."""
+    from safetensors.torch import load_file, save_file
+
+    from symmetry_amd.models.weights import random_weights
+
+    c = C.resolve("tiny-komazen")
+    eng = LLMEngine(EngineConfig(model="tiny-komazen", weights="random", dtype="float32", device="cpu", max_num_seqs=2,
+                                 block_size=16, num_kv_blocks=9, max_model_len=128, use_graphs=False,
+                                 enable_prefix_caching=False, pipeline=False, seed=3))
+    W = {k: v.to(torch.bfloat16) for k, v in random_weights(c, seed=3).tensors.items()}
+    toks = tokens(50, c.vocab_size, 2)
+    got = run_schedule(eng, {"a": toks}, [[("a", 31)], [("a", 19)]])["a"]
+    assert err(got, oracle_logits(C.komazen_to_config(c), W, toks)) < TOL["float32"]
+    cfg = cfg_mixed()
+    path, cj, W = checkpoint(cfg, tmp_path, seed=4)
+    f = os.path.join(path, "model.safetensors")
+    t = load_file(f)
+    t["l2.norm2"], t["l2.canon2"] = torch.ones(cfg.hidden_size), torch.zeros(cfg.hidden_size, cfg.conv_taps)
+    save_file(t, f)
+    toks = tokens(20, cfg.vocab_size, 5)
+    got = run_schedule(engine(path, "cpu", "float32"), {"a": toks}, [[("a", 20)]])["a"]
+    assert err(got, oracle_logits(cj, W, toks)) < TOL["float32"]
+    t["l2.sink"] = torch.zeros(3)
+    save_file(t, f)
+    with pytest.raises(ValueError):
+        engine(path, "cpu", "float32")
+
+
 # ---- mechanisms alone: op against oracle function ---------------------------------------------------------------
 def _dev(device, *ts):
     return [t.to(device) if torch.is_tensor(t) else t for t in ts]
