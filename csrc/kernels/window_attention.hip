@@ -117,9 +117,11 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
       slot = cache_row(bt, j, a.BS, a.bs_shift);
       dot_rows<T, REP>(kc + (slot * a.G + g) * a.dk, qs, a.dk, sc);
       if (a.bias) {
+        // (the 32-bit model takes log1pf; bf16 activations the hardware logarithm, whose error is far below their rounding)
         const float dist = (float)(p - j);
 #pragma unroll
-        for (int r = 0; r < REP; ++r) sc[r] -= b1[r] * log1pf(b2[r] * dist);
+        for (int r = 0; r < REP; ++r)
+          sc[r] -= b1[r] * (sizeof(T) == 4 ? log1pf(b2[r] * dist) : __logf(1.f + b2[r] * dist));
       }
     }
 #pragma unroll
@@ -353,6 +355,8 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
     const bool interior = 16 * wave + 15 < nrows && kt + 63 <= wq_lo && kt > wq_hi - a.window;
     float pv[4][4];
     float mx = -INFINITY;
+    // 1 + b2 (qp - kp) for key kp = kt + 16 s4 + 4 hq + e is arg0 - b2 (16 s4 + e): one multiply-add per score
+    const float arg0 = 1.f + b2 * (float)(qp - kt - 4 * hq), nb1 = -b1;
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -366,7 +370,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           pv[s4][e] = acc[e] * sl2;
-          if (biased) pv[s4][e] -= b1 * __log2f(1.f + b2 * (float)(qp - (kt + 16 * s4 + 4 * hq + e)));
+          if (biased) pv[s4][e] += nb1 * __log2f(arg0 - b2 * (float)(16 * s4 + e));
           mx = fmaxf(mx, pv[s4][e]);
         }
       } else {
@@ -375,7 +379,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
           const int kp = kt + 16 * s4 + 4 * hq + e;
           const bool vis = rv && kp <= qp && kp > qp - a.window;
           float sv = acc[e] * sl2;
-          if (biased) sv -= b1 * __log2f(1.f + b2 * (float)max(qp - kp, 0));
+          if (biased) sv += nb1 * __log2f(arg0 - b2 * (float)(16 * s4 + e));   // (keys past the row: masked below)
           pv[s4][e] = vis ? sv : -INFINITY;
           mx = fmaxf(mx, pv[s4][e]);
         }
