@@ -15,6 +15,10 @@ def model_class(cfg):
         from .komazen import KomazenLM
 
         return KomazenLM
+    if family == "dalalix":
+        from .dalalix import DalalixLM
+
+        return DalalixLM
     if family == "llama":
         from .transformer import TransformerLM
 

@@ -274,6 +274,7 @@ class RotarySpec:
     original: float = 0.0
     fast: float = 0.0
     slow: float = 0.0
+    half: bool = False           # True: entry i turns with entry i + dims / 2 (half layout) instead of the pairs (2i, 2i + 1)
 
 
 @dataclass(frozen=True)
@@ -285,6 +286,10 @@ class WindowAttnSpec:
     window: int                  # a position sees itself and the window - 1 positions before it
     scale: float
     rot: RotarySpec
+    keep_first: int = 0          # the sequence's first positions stay visible past the window (at their true positions)
+    sink: bool = False           # a learned per-head logit in the softmax's denominator (no key, no value)
+    gate: bool = True            # per-head sigmoid output gate
+    out_bias: bool = True        # bias on the output projection
 
 
 @dataclass(frozen=True)
@@ -726,6 +731,275 @@ TINY_KOMAZEN = komazen_stack("tiny-komazen", 512, 128, "LASA", heads=4, kv_heads
 SMALL_KOMAZEN = komazen_stack("small-komazen", 32768, 2048, "LASA", heads=16, kv_heads=4, dim=128, ff=8192, window=1024,
                               max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
 
+# --------------------------------------------------------------------------------------------------
+# Dalalix: several residual streams mixed by learned matrices (hyper-connections) around pre-norm sublayers; the token
+# embedding plus a hashed (previous token, token) embedding; layers that borrow another layer's weights; mixers: causal
+# grouped-head attention (biased projections, or a short convolution on q / k / v + unit-RMS values + an element-wise
+# output gate), or windowed attention with kept first tokens and a sink beside a matrix memory with exponential gating;
+# routed clamped-GLU experts with group-limited choice; soft-capped logits.
+# --------------------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class HashPairSpec:
+    """Row (prev * mul_prev + tok * mul_cur) mod buckets of a [buckets + 1, width] table; a sequence's first token takes
+    the last row."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+
+@dataclass(frozen=True)
+class CausalAttnSpec:
+    """Causal softmax attention with grouped key / value heads and no positions in the scores."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    bias: bool = False           # q / k / v projections carry biases
+    conv: int = 0                # taps of the causal per-channel convolution on q, k and v (0: none)
+    v_norm: bool = False         # values are brought to unit RMS per head before they are cached
+    gate: bool = False           # element-wise sigmoid(W_g h) on the concatenated heads
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """Matrix memory with exponential input gate, sigmoid forget gate (both soft-capped) and a running maximum."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+@dataclass(frozen=True)
+class GroupRoutedSpec:
+    """Softmax router; experts in ``groups`` equal groups of neighbours, only the ``keep`` best groups (by their best
+    expert) are eligible; weights = chosen scores over their sum; clamped-GLU experts."""
+    experts: int
+    top: int
+    expert_ff: int
+    limit: float
+    groups: int = 1
+    keep: int = 1
+
+
+@dataclass(frozen=True)
+class DalalixLayer:
+    type: str                    # "attention" | "attention_2" | "parallel"
+    mixer: CausalAttnSpec | PairMixerSpec
+    mlp: GroupRoutedSpec | None = None
+    weights_of: int | None = None   # the layer whose tensors this one reads (cache and state stay its own)
+
+
+@dataclass(frozen=True)
+class DalalixConfig:
+    family = "dalalix"
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    streams: int = 0             # residual streams; 0: the plain residual sum (no mixing tensors)
+    bigram: HashPairSpec | None = None
+    logit_softcap: float = 0.0   # 0: none
+    norm_eps: float = 1e-5
+    max_position: int = 131072
+    bos_token_id: int = 1
+    eos_token_ids: tuple = (2,)
+    chat_format: str = "llama3"
+    tie_embeddings = False
+    rope_scaling = None
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(layer.mlp is not None for layer in self.layers)
+
+    def owner(self, i: int) -> int:
+        """The layer whose tensors layer i reads."""
+        w = self.layers[i].weights_of
+        return i if w is None else w
+
+    def attn_spec(self, i: int):
+        """The softmax-attention part of layer i's mixer (every layer has one)."""
+        layer = self.layers[i]
+        return layer.mixer.left if layer.type == "parallel" else layer.mixer
+
+    def num_params(self) -> int:
+        from .weights import dalalix_shapes
+
+        n = 0
+        for shape in dalalix_shapes(self).values():
+            k = 1
+            for v in shape:
+                k *= v
+            n += k
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum(a.kv_heads * (a.dim + a.vdim) for a in map(self.attn_spec, range(self.num_layers))) * dtype_bytes
+
+    def state_bytes_per_seq(self, dtype_bytes: int = 2) -> int:
+        n = 4 if self.bigram else 0
+        for layer in self.layers:
+            m = layer.mixer
+            if layer.type == "parallel":
+                n += m.right.heads * (m.right.dim * (m.right.vdim + 1) + 1) * 4
+            elif m.conv > 1:
+                n += (m.conv - 1) * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) * dtype_bytes
+        return n
+
+    def replace(self, **kw) -> "DalalixConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def dalalix_from_config(cfg: dict, name: str = "dalalix") -> DalalixConfig:
+    """config.json of a Dalalix checkpoint: every size and constant is read here; a key this reader does not know means
+    a mechanism this code does not have, so it raises."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        kind, mixer, mlp, wof = _take(L, f"layer {i}", "type", "mixer", optional=("mlp", "weights_of"))
+        if kind in ("attention", "attention_2"):
+            dim, heads, kvh, scale, vdim, conv = _take(mixer, f"layer {i} mixer", "dim", "heads", "kv_heads", "scale",
+                                                       "vdim", optional=("conv",))
+            if (kind == "attention") != (conv is not None):
+                raise ValueError(f"layer {i}: {kind!r} and conv = {conv!r} do not fit")
+            plain = kind == "attention_2"
+            mix = CausalAttnSpec(int(heads), int(kvh), int(dim), int(vdim), float(scale), bias=plain,
+                                 conv=0 if plain else int(conv), v_norm=not plain, gate=not plain)
+            if mix.heads % mix.kv_heads or (not plain and not 1 <= mix.conv <= 16):
+                raise ValueError(f"layer {i}: heads {heads} / kv_heads {kvh} / conv {conv} do not fit")
+        elif kind == "parallel":
+            left, right, ls, rs = _take(mixer, f"layer {i} mixer", "left", "right", "left_scale", "right_scale")
+            dim, heads, kvh, mask, rot, scale, vdim = _take(left, f"layer {i} left", "dim", "heads", "kv_heads", "mask",
+                                                            "rot", "scale", "vdim")
+            window, keep = _take(mask, f"layer {i} mask", "size", optional=("keep_first",))
+            base, dims = _take(rot, f"layer {i} rot", "base", "dims")
+            lspec = WindowAttnSpec(int(heads), int(kvh), int(dim), int(vdim), int(window), float(scale),
+                                   RotarySpec(int(dims), float(base), half=True), keep_first=int(keep or 0), sink=True,
+                                   gate=False, out_bias=False)
+            if lspec.heads % lspec.kv_heads or lspec.rot.dims % 2 or lspec.rot.dims > lspec.dim or lspec.window < 1 \
+                    or lspec.keep_first < 0:
+                raise ValueError(f"layer {i}: heads {heads} / kv_heads {kvh} / rot.dims {dims} / dim {dim} / mask do not fit")
+            rdim, cap, rheads, rvdim = _take(right, f"layer {i} right", "dim", "gate_cap", "heads", "vdim")
+            mix = PairMixerSpec(lspec, MatrixMemorySpec(int(rheads), int(rdim), int(rvdim), float(cap)), float(ls), float(rs))
+        else:
+            raise ValueError(f"layer {i}: unknown layer type {kind!r}")
+        if mlp is None:
+            ff = None
+        elif mlp.get("kind") == "moe":
+            _, expert, router = _take(mlp, f"layer {i} mlp", "kind", "expert", "router")
+            eff, limit = _take(expert, f"layer {i} mlp.expert", "ff", "limit")
+            experts, top, groups = _take(router, f"layer {i} mlp.router", "experts", "top", optional=("groups",))
+            count, keep = _take(groups, f"layer {i} mlp.router.groups", "count", "keep") if groups else (1, 1)
+            ff = GroupRoutedSpec(int(experts), int(top), int(eff), float(limit), int(count), int(keep))
+            if ff.experts % ff.groups or not 1 <= ff.keep <= ff.groups or not 1 <= ff.top <= ff.keep * (ff.experts // ff.groups):
+                raise ValueError(f"layer {i}: top {top} of {experts} experts in {count} groups, {keep} kept")
+        else:
+            raise ValueError(f"layer {i}: unknown mlp kind {mlp.get('kind')!r}")
+        layer = DalalixLayer(kind, mix, ff, None if wof is None else int(wof))
+        if layer.weights_of is not None:
+            src = layers[layer.weights_of] if 0 <= layer.weights_of < i else None
+            if src is None or src.weights_of is not None or (src.type, src.mixer, src.mlp) != (kind, mix, ff):
+                raise ValueError(f"layer {i}: weights_of {wof} must name an earlier layer of the same sizes with tensors "
+                                 "of its own")
+        layers.append(layer)
+    vocab, width, norm, _, _, emb, streams, cap, bos, eos = _take(
+        cfg, "config", "vocab", "width", "norm", "layers",
+        optional=("architecture", "embedding", "streams", "logit_softcap", "bos_token_id", "eos_token_ids"))
+    (eps,) = _take(norm, "norm", "eps")
+    (bg,) = _take(emb, "embedding", optional=("bigram",)) if emb else (None,)
+    if bg:
+        buckets, mc, mp = _take(bg, "embedding.bigram", "buckets", "mul_cur", "mul_prev")
+        bg = HashPairSpec(int(buckets), int(mp), int(mc))
+        if bg.buckets < 1:
+            raise ValueError("embedding.bigram.buckets < 1")
+    return DalalixConfig(name=name, vocab_size=int(vocab), hidden_size=int(width), layers=tuple(layers),
+                         streams=int(streams or 0), bigram=bg or None, logit_softcap=float(cap or 0.0),
+                         norm_eps=float(eps), bos_token_id=int(bos if bos is not None else 1),
+                         eos_token_ids=tuple(eos) if eos is not None else (2,))
+
+
+def dalalix_to_config(c: DalalixConfig) -> dict:
+    """The config.json form of a DalalixConfig (exports, tests)."""
+    layers = []
+    for layer in c.layers:
+        m = layer.mixer
+        if layer.type == "parallel":
+            a, g = m.left, m.right
+            md = {"left": {"dim": a.dim, "heads": a.heads, "kv_heads": a.kv_heads,
+                           "mask": {"keep_first": a.keep_first, "size": a.window},
+                           "rot": {"base": a.rot.base, "dims": a.rot.dims}, "scale": a.scale, "vdim": a.vdim},
+                  "left_scale": m.left_scale,
+                  "right": {"dim": g.dim, "gate_cap": g.gate_cap, "heads": g.heads, "vdim": g.vdim},
+                  "right_scale": m.right_scale}
+        else:
+            md = {"dim": m.dim, "heads": m.heads, "kv_heads": m.kv_heads, "scale": m.scale, "vdim": m.vdim}
+            if layer.type == "attention":
+                md["conv"] = m.conv
+        f = layer.mlp
+        fd = None if f is None else {"expert": {"ff": f.expert_ff, "limit": f.limit}, "kind": "moe",
+                                     "router": {"experts": f.experts, "groups": {"count": f.groups, "keep": f.keep},
+                                                "top": f.top}}
+        d = {"mixer": md, "mlp": fd, "type": layer.type}
+        if layer.weights_of is not None:
+            d["weights_of"] = layer.weights_of
+        layers.append(d)
+    out = {"architecture": "Dalalix", "layers": layers, "norm": {"eps": c.norm_eps}, "vocab": c.vocab_size,
+           "width": c.hidden_size}
+    if c.bigram:
+        out["embedding"] = {"bigram": {"buckets": c.bigram.buckets, "mul_cur": c.bigram.mul_cur,
+                                       "mul_prev": c.bigram.mul_prev}}
+    if c.streams:
+        out["streams"] = c.streams
+    if c.logit_softcap:
+        out["logit_softcap"] = c.logit_softcap
+    return out
+
+
+def dalalix_stack(name, vocab, width, pattern, heads, kv_heads, dim, experts, top, expert_ff, window=1024, keep_first=4,
+                  rot_dims=None, vdim=None, mem_heads=None, mem_dim=None, mem_vdim=None, conv=4, groups=1, keep=1,
+                  limit=7.0, streams=4, buckets=0, softcap=30.0, **kw) -> DalalixConfig:
+    """A stack from a pattern string: "B" causal attention with biased projections, "C" causal attention with the short
+    convolution, unit-RMS values and the output gate, "P" windowed attention beside the matrix memory; a digit repeats
+    the layer with that index with its weights (cache and state its own); lower case = no feed-forward."""
+    vdim = vdim or dim
+    layers = []
+    for ch in pattern:
+        if ch.isdigit():
+            src = layers[int(ch)]
+            layers.append(dataclasses.replace(src, weights_of=int(ch)))
+            continue
+        if ch in "Bb":
+            kind, mix = "attention_2", CausalAttnSpec(heads, kv_heads, dim, vdim, dim ** -0.5, bias=True)
+        elif ch in "Cc":
+            kind, mix = "attention", CausalAttnSpec(heads, kv_heads, dim, vdim, dim ** -0.5, conv=conv, v_norm=True,
+                                                    gate=True)
+        elif ch in "Pp":
+            left = WindowAttnSpec(heads, kv_heads, dim, vdim, window, dim ** -0.5,
+                                  RotarySpec(rot_dims or dim // 2, 10000.0, half=True), keep_first=keep_first, sink=True,
+                                  gate=False, out_bias=False)
+            right = MatrixMemorySpec(mem_heads or heads, mem_dim or dim, mem_vdim or vdim, 15.0)
+            kind, mix = "parallel", PairMixerSpec(left, right, 0.5, 0.5)
+        else:
+            raise ValueError(f"pattern letter {ch!r}")
+        mlp = GroupRoutedSpec(experts, top, expert_ff, limit, groups, keep) if ch.isupper() else None
+        layers.append(DalalixLayer(kind, mix, mlp))
+    bg = HashPairSpec(buckets, 1000003, 31) if buckets else None
+    return DalalixConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), streams=streams, bigram=bg,
+                         logit_softcap=softcap, **kw)
+
+
+TINY_DALALIX = dalalix_stack("tiny-dalalix", 512, 128, "BPC1", heads=4, kv_heads=2, dim=32, experts=6, top=2, expert_ff=64,
+                             window=48, keep_first=3, rot_dims=16, mem_heads=2, mem_dim=16, mem_vdim=32, conv=3, groups=3,
+                             keep=2, limit=3.0, streams=3, buckets=251, max_position=2048, bos_token_id=500,
+                             eos_token_ids=(501, 502))
+# layer shapes of a mid-size model (benchmarks; random weights)
+SMALL_DALALIX = dalalix_stack("small-dalalix", 32768, 2048, "BPCC", heads=16, kv_heads=4, dim=128, experts=16, top=4,
+                              expert_ff=1024, window=1024, mem_heads=8, mem_dim=128, mem_vdim=256, groups=4, keep=2,
+                              buckets=65521, max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+
 LLAMA31_SCALING = {
     "rope_type": "llama3",
     "factor": 8.0,
@@ -768,7 +1042,7 @@ _REGISTRY = {
     c.name: c
     for c in (LLAMA3_8B, LLAMA31_8B, LLAMA3_70B, LLAMA31_70B, MIXTRAL_8X7B, TINY_LLAMA, TINY_MIXTRAL, SMALL_LLAMA,
               TINY_LLAMA_KV8, TINY_MIXTRAL_E8, TINY_BOZEVIK, SMALL_BOZEVIK, SMALL_BOZEVIK_MOE, TINY_LEMUNEX,
-              SMALL_LEMUNEX, SMALL_LEMUNEX_MOE, TINY_KOMAZEN, SMALL_KOMAZEN)
+              SMALL_LEMUNEX, SMALL_LEMUNEX_MOE, TINY_KOMAZEN, SMALL_KOMAZEN, TINY_DALALIX, SMALL_DALALIX)
 }
 _ALIASES = {
     "llama3": "llama3:8b",
@@ -801,7 +1075,7 @@ def known_models() -> list[str]:
 
 def from_config_json(cfg: dict, name: str = "hf", shapes: dict | None = None):
     """The model configuration of a checkpoint directory's config.json: the design is chosen by its
-    ``architecture`` key (Bozevik, Lemunex, Komazen), otherwise the HuggingFace Llama / Mixtral keys.  ``shapes``: the
+    ``architecture`` key (Bozevik, Lemunex, Komazen, Dalalix), otherwise the HuggingFace Llama / Mixtral keys.  ``shapes``: the
     checkpoint's tensor shapes, for designs that leave some sizes to them."""
     if cfg.get("architecture") == "Bozevik":
         return bozevik_from_config(cfg, name)
@@ -809,6 +1083,8 @@ def from_config_json(cfg: dict, name: str = "hf", shapes: dict | None = None):
         return lemunex_from_config(cfg, name, shapes)
     if cfg.get("architecture") == "Komazen":
         return komazen_from_config(cfg, name)
+    if cfg.get("architecture") == "Dalalix":
+        return dalalix_from_config(cfg, name)
     return from_hf_config(cfg, name)
 
 

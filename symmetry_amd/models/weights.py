@@ -184,6 +184,8 @@ def random_weights(cfg: ModelConfig, shard: ShardSpec | None = None, device="cpu
         return lemunex_random_weights(cfg, shard, device, dtype, seed)
     if getattr(cfg, "family", "llama") == "komazen":
         return komazen_random_weights(cfg, shard, device, dtype, seed)
+    if getattr(cfg, "family", "llama") == "dalalix":
+        return dalalix_random_weights(cfg, shard, device, dtype, seed)
     shard.validate(cfg)
     shapes = full_shapes(cfg)
     tensors = {}
@@ -242,6 +244,8 @@ def load_hf_weights(path: str, cfg: ModelConfig, shard: ShardSpec | None = None,
         return load_lemunex_weights(path, cfg, shard, device, dtype)
     if getattr(cfg, "family", "llama") == "komazen":
         return load_komazen_weights(path, cfg, shard, device, dtype)
+    if getattr(cfg, "family", "llama") == "dalalix":
+        return load_dalalix_weights(path, cfg, shard, device, dtype)
     shard.validate(cfg)
     wmap = _hf_index(path)
     handles = {}
@@ -648,5 +652,141 @@ def save_komazen_checkpoint(weights: ModelWeights, path: str) -> None:
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(komazen_to_config(weights.cfg), f, indent=1)
+    save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
+              os.path.join(path, "model.safetensors"))
+
+
+# --------------------------------------------------------------------------------------------------
+# Dalalix checkpoints: tensors keep the checkpoint's names (embed, bigram, l<i>.norm1, l<i>.hc1.in, l<i>.mix.q,
+# l<i>.mix.left.sink, l<i>.mix.right.i, l<i>.mlp.e<j>.gate, ..., final.norm, head); a layer that borrows another's
+# weights has no tensors.  models/dalalix.py fuses what its GEMMs read.
+# --------------------------------------------------------------------------------------------------
+def dalalix_shapes(cfg, optional: set | None = None) -> dict:
+    """Tensor name -> shape.  ``optional`` (a set) receives the names a checkpoint may carry without this code reading
+    them: the second norm and stream mixing of a layer that has no feed-forward."""
+    d, S = cfg.hidden_size, cfg.streams
+    shapes = {"embed": (cfg.vocab_size, d), "final.norm": (d,), "head": (cfg.vocab_size, d)}
+    if cfg.bigram:
+        shapes["bigram"] = (cfg.bigram.buckets + 1, d)
+    for i, layer in enumerate(cfg.layers):
+        if layer.weights_of is not None:
+            continue
+        p, m = f"l{i}.", layer.mixer
+        subs = {1: True, 2: layer.mlp is not None}
+        for q, there in subs.items():
+            names = {f"{p}norm{q}": (d,)}
+            if S:
+                names.update({f"{p}hc{q}.in": (S,), f"{p}hc{q}.out": (S,), f"{p}hc{q}.mix": (S, S)})
+            if there:
+                shapes.update(names)
+            elif optional is not None:
+                optional.update(names)
+        if layer.type == "parallel":
+            a, g, q = m.left, m.right, p + "mix."
+            for nm, rows in (("q", a.heads * a.dim), ("k", a.kv_heads * a.dim), ("v", a.kv_heads * a.vdim)):
+                shapes[f"{q}left.{nm}"], shapes[f"{q}left.{nm}.b"] = (rows, d), (rows,)
+            shapes[q + "left.sink"] = (a.heads,)
+            shapes[q + "left.o"] = (d, a.heads * a.vdim)
+            shapes[q + "right.q"] = shapes[q + "right.k"] = (g.heads * g.dim, d)
+            shapes[q + "right.v"] = shapes[q + "right.g"] = (g.heads * g.vdim, d)
+            shapes[q + "right.o"] = (d, g.heads * g.vdim)
+            shapes[q + "right.norm"] = (g.heads * g.vdim,)
+            for nm in ("i", "f"):
+                shapes[f"{q}right.{nm}"], shapes[f"{q}right.{nm}.b"] = (g.heads, d), (g.heads,)
+        else:
+            q = p + "mix."
+            for nm, rows in (("q", m.heads * m.dim), ("k", m.kv_heads * m.dim), ("v", m.kv_heads * m.vdim)):
+                shapes[q + nm] = (rows, d)
+                if m.bias:
+                    shapes[f"{q}{nm}.b"] = (rows,)
+                if m.conv:
+                    shapes[f"{q}{nm}.conv"] = (rows, m.conv)
+            if m.gate:
+                shapes[q + "g"] = (m.heads * m.vdim, d)
+            shapes[q + "o"] = (d, m.heads * m.vdim)
+        f = layer.mlp
+        if f is not None:
+            for e in range(f.experts):
+                shapes[f"{p}mlp.e{e}.gate"] = shapes[f"{p}mlp.e{e}.up"] = (f.expert_ff, d)
+                shapes[f"{p}mlp.e{e}.down"] = (d, f.expert_ff)
+            shapes[p + "mlp.router"] = (f.experts, d)
+    return shapes
+
+
+def dalalix_random_weights(cfg, shard: ShardSpec | None = None, device="cpu", dtype=torch.bfloat16,
+                           seed: int = 0) -> ModelWeights:
+    """Random init (benchmarks, tests): matrices N(0, (1.28 / sqrt(fan_in))^2); norm weights around one; stream mixing
+    near a permutation-free average with every entry nonzero; biases, sinks and convolution taps nonzero; forget-gate
+    biases high enough that the memory remembers hundreds of tokens -- all away from the values at which a dropped
+    parameter would not show."""
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Dalalix runs on one GPU per replica (its tensors are not sharded)")
+    tensors = {}
+    S = max(cfg.streams, 1)
+    for name, shape in dalalix_shapes(cfg).items():
+        g = torch.Generator().manual_seed(_seed(seed, name))
+        leaf = name.rsplit(".", 1)[-1]
+        if leaf in ("norm", "norm1", "norm2"):
+            t = 0.75 + 0.5 * torch.rand(shape, generator=g)
+        elif name.endswith(".mix") and ".hc" in name:
+            t = torch.eye(S) * 0.7 + 0.3 / S + 0.1 * torch.randn(shape, generator=g)
+        elif leaf == "in" and ".hc" in name:
+            t = 1.0 / S + 0.2 * torch.randn(shape, generator=g)
+        elif leaf == "out" and ".hc" in name:
+            t = 1.0 / S + 0.3 * torch.rand(shape, generator=g)
+        elif name.endswith("right.f.b"):
+            t = 3.0 + torch.randn(shape, generator=g)
+        elif name.endswith("right.i.b"):
+            t = -1.0 + torch.randn(shape, generator=g)
+        elif leaf == "sink":
+            t = torch.randn(shape, generator=g)
+        elif leaf == "b":
+            t = 0.2 * torch.randn(shape, generator=g)
+        elif leaf == "conv":
+            t = torch.randn(shape, generator=g) * shape[1] ** -0.5
+        elif name == "bigram":
+            t = torch.randn(shape, generator=g)
+        else:
+            tensors[name] = _randn(shape, _seed(seed, name), device, dtype, 1.0 if name == "embed" else _std(name, shape))
+            continue
+        tensors[name] = t.to(dtype).to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def load_dalalix_weights(path: str, cfg, shard: ShardSpec | None = None, device="cpu",
+                         dtype=torch.bfloat16) -> ModelWeights:
+    """model.safetensors of a Dalalix checkpoint directory; every tensor the configuration implies must be there with
+    the implied shape, and no other.  Tensors stay in the file's precision (the model converts what it fuses)."""
+    from safetensors import safe_open
+
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Dalalix runs on one GPU per replica (its tensors are not sharded)")
+    optional: set = set()
+    shapes = dalalix_shapes(cfg, optional)
+    tensors = {}
+    with safe_open(os.path.join(path, "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+        missing, extra = sorted(set(shapes) - names), sorted(names - set(shapes) - optional)
+        if missing or extra:
+            raise ValueError(f"checkpoint does not fit its config: missing {missing[:4]}, unexpected {extra[:4]}")
+        for name, shape in shapes.items():
+            t = f.get_tensor(name)
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"{name}: shape {tuple(t.shape)}, the config implies {tuple(shape)}")
+            tensors[name] = t.to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def save_dalalix_checkpoint(weights: ModelWeights, path: str) -> None:
+    """config.json + model.safetensors (bf16) of a Dalalix model, in the form the loader reads."""
+    from safetensors.torch import save_file
+
+    from .config import dalalix_to_config
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(dalalix_to_config(weights.cfg), f, indent=1)
     save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
               os.path.join(path, "model.safetensors"))

@@ -750,52 +750,69 @@ def rope_scaled_table(max_pos, dims, base, factor=0.0, original=0.0, fast=0.0, s
     return reference.rope_scaled_table(max_pos, dims, base, factor, original, fast, slow, device)
 
 
-def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache):
-    """z [T, H dk | G dk | G dv (| ...)] + bias (fp32) -> q_out [T, H, dk] and the token's rows of the paged caches
-    k [NB, BS, G, dk], v [NB, BS, G, dv] (slot >= 0); q and k turn by ``rope`` [max_pos, pairs, 2] on their first
-    2 * pairs entries (interleaved pairs), in fp32."""
+def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache, half_dims=0):
+    """z [T, H dk | G dk | G dv (| ...)] + bias (fp32, optional) -> q_out [T, H, dk] and the token's rows of the paged
+    caches k [NB, BS, G, dk], v [NB, BS, G, dv] (slot >= 0); q and k turn by ``rope`` [max_pos, pairs, 2] (optional) on
+    their first 2 * pairs entries, in fp32: interleaved pairs (2i, 2i + 1), or with ``half_dims`` = 2 * pairs the half
+    layout (entry i with entry i + pairs)."""
     if _gpu(z):
         return _hyb().qkv_rope_cache(z, bias, int(H), int(G), int(dk), int(dv), positions, slots, rope, q_out,
-                                     k_cache, v_cache)
-    return reference.qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache)
+                                     k_cache, v_cache, int(half_dims))
+    return reference.qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache, half_dims)
 
 
 WINDOW_ATTN_IMPL = 0 if os.environ.get("SYMMETRY_WINDOW_ATTN", "auto") == "wave" else 1  # A/B: the all-shapes kernel
 
 
 def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, tiles=None, cu_q=None,
-                impl=None, bias=None):
+                impl=None, bias=None, keep_first=0, sink=None):
     """Softmax attention of q [T, H, dk] over the paged caches: row r sees positions max(0, p - window + 1) .. p of
-    sequence row_seq[r] (p = positions[r]); query head h reads key / value head h // (H / G); scores and weights
-    fp32.  ``gate`` [T, H] (a view): head outputs are multiplied by sigmoid(gate).  ``tiles`` / ``cu_q``: the packed
-    prompt form (64-row query tiles), for the tiled kernel.  Returns the implementation used (0: one wave per (row,
-    head), every shape; 1: tiled).  ``bias`` [2, H] fp32: the score of a key at distance n = p - j is lowered by
-    bias[0, h] * ln(1 + bias[1, h] * n)."""
+    sequence row_seq[r] (p = positions[r]) and, with ``keep_first``, the sequence's first keep_first positions; query
+    head h reads key / value head h // (H / G); scores and weights fp32.  ``gate`` [T, H] (a view): head outputs are
+    multiplied by sigmoid(gate).  ``tiles`` / ``cu_q``: the packed prompt form (64-row query tiles), for the tiled
+    kernel.  Returns the implementation used (0: one wave per (row, head), every shape; 1: tiled).  ``bias`` [2, H] fp32:
+    the score of a key at distance n = p - j is lowered by bias[0, h] * ln(1 + bias[1, h] * n).  ``sink`` [H] fp32: the
+    softmax's denominator of head h also holds exp(sink[h]) (a logit without a key or a value, not scaled)."""
     if _gpu(q):
         return _hyb().window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, int(window), float(scale), gate,
-                                  out, tiles, cu_q, WINDOW_ATTN_IMPL if impl is None else int(impl), bias)
-    reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias)
+                                  out, tiles, cu_q, WINDOW_ATTN_IMPL if impl is None else int(impl), bias,
+                                  int(keep_first), sink)
+    reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias,
+                          keep_first, sink)
     return 0
 
 
-DECAY_CHANNEL_GATE, DECAY_STEP_SIZE = 0, 1
+DECAY_CHANNEL_GATE, DECAY_STEP_SIZE, DECAY_LOG_GATES = 0, 1, 2
 
 
 def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
-               out):
+               out, mstate=None, mout=None):
     """Linear recurrence with decaying state, per head h over every run of rows (cu_q[i] .. cu_q[i + 1]; cu_q None:
     every row its own run): S <- diag(a_t) S + b_t k_t v_t^T (S [N, P] fp32), out_t = S^T (q_scale q_t) (+ skip_h v_t).
     DECAY_CHANNEL_GATE: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel (dz [T, H N], dparam a number), b = 1;
     DECAY_STEP_SIZE: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) b) per head (dz [T, H]).
+    DECAY_LOG_GATES: dz fp32 [T, 2 H] = input | forget pre-activations, dbias [2 H], dparam the gates' soft cap c:
+    i = c tanh(. / c), f = logsigmoid(c tanh(. / c)), running maximum m_t = max(f + m_(t-1), i) (0 at a sequence's start,
+    carried in mstate [slots, H], written to mout [T, H]), a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); state
+    [slots, H, N, P + 1] and out [T, H, P + 1] carry one more column, fed by v = 1 (the normaliser n_t and n_t . q_t).
     q / k [T, (H / hpg) N]: head h reads group h // hpg.  A run starts from state[slot] if prev_row[first] <= -2
     (slot = -(v + 2)), else from zero; it ends in state[save_slot[last]] (>= 0).  out fp32 [T, H, P]."""
     if _gpu(out):
         dp = dparam if torch.is_tensor(dparam) else None
         return _hyb().decay_scan(int(mode), q, k, v, dz, dbias, dp, 0.0 if dp is not None else float(dparam), skip,
                                  float(q_scale), int(H), int(N), int(P), int(hpg), state, cu_q, prev_row, save_slot,
-                                 int(runs), out)
+                                 int(runs), out, mstate, mout)
     return reference.decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row,
-                                save_slot, runs, out)
+                                save_slot, runs, out, mstate, mout)
+
+
+def memory_norm_gate(y, m, gate, w, eps, out):
+    """Read-out of a matrix memory (``decay_scan`` with DECAY_LOG_GATES): y fp32 [T, H, P + 1] whose last column is
+    n . q, m fp32 [T, H]: o = y[..., :P] / (max(|n . q|, exp(-m)) + 1e-6), each head brought to unit RMS (eps), times
+    w [H P], times sigmoid(gate) (gate [T, H P], a view) -> out [T, H P]."""
+    if _gpu(y):
+        return _hyb().memory_norm_gate(y, m, gate, w, float(eps), out)
+    return reference.memory_norm_gate(y, m, gate, w, eps, out)
 
 
 def gated_group_norm(y, gate, w, eps, group, gate_first, out):
@@ -835,11 +852,14 @@ def silu_mul(gate, up, out):
     return reference.silu_mul(gate, up, out)
 
 
-def softmax_topk(x, Wr, corr, k, ids, w):
-    """Router: s = softmax(x @ Wr.T) in fp32 over all outputs; the k largest of s + corr -> ids [T, k]; w = their s."""
+def softmax_topk(x, Wr, corr, k, ids, w, groups=1, keep=1, renorm=False):
+    """Router: s = softmax(x @ Wr.T) in fp32 over all outputs; the k largest of s + corr (corr optional) -> ids [T, k];
+    w = their s, with ``renorm`` divided by their sum (+ 1e-20).  ``groups`` / ``keep``: the outputs form ``groups``
+    equal groups of neighbours, a group scores as its largest entry, and only entries of the ``keep`` best groups can be
+    chosen."""
     if _gpu(x):
-        return _hyb().softmax_topk(x, Wr, corr, int(k), ids, w)
-    return reference.softmax_topk(x, Wr, corr, k, ids, w)
+        return _hyb().softmax_topk(x, Wr, corr, int(k), ids, w, int(groups), int(keep), bool(renorm))
+    return reference.softmax_topk(x, Wr, corr, k, ids, w, groups, keep, renorm)
 
 
 def moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out):
@@ -926,3 +946,73 @@ def sigmoid_mul(a, gate, out):
     if _gpu(out):
         return _hyb().sigmoid_mul(a, gate, out)
     return reference.sigmoid_mul(a, gate, out)
+
+
+# ---- several residual streams, hashed token pairs, convolved projections (csrc/kernels/hybrid_rows.hip) -----------
+def embed_pair_hash(ids, table, pair_table, buckets, mul_prev, mul_cur, prev_row, tok_state, x, save_slot=None, src=None,
+                    prev=None):
+    """x fp32 [T, S, d]: every one of the S streams = table[token] + pair_table[(p * mul_prev + token * mul_cur) mod
+    buckets], p the sequence's previous token: the row prev_row[r] of this step (>= 0), the carried token
+    tok_state[-(prev_row[r] + 2)] (<= -2), or none (-1: the table's extra row ``buckets``).  ``pair_table`` None: the
+    token rows alone.  Rows with src >= 0 take the token prev[src] (the previous step's sample, still on the device).
+    ``save_slot`` (steps whose rows are runs of their own): the row's token becomes the carried one; otherwise
+    ``token_state_update`` stores it."""
+    if _gpu(x):
+        return _hyb().embed_pair_hash(ids, src, prev, table, pair_table, int(buckets), int(mul_prev), int(mul_cur),
+                                      prev_row, tok_state, save_slot, x)
+    tok = reference.resolve_ids(ids, src, prev)
+    reference.embed_pair_hash(tok, table, pair_table, buckets, mul_prev, mul_cur, prev_row, tok_state, x)
+    if save_slot is not None:
+        reference.token_state_update(tok[:x.shape[0]], tok_state, None, save_slot, x.shape[0])
+
+
+def token_state_update(ids, tok_state, cu_q, save_slot, runs):
+    """tok_state[save_slot[last]] = the last token of every run (cu_q[i] .. cu_q[i + 1])."""
+    if _gpu(ids):
+        return _hyb().token_state_update(ids, tok_state, cu_q, save_slot, int(runs))
+    return reference.token_state_update(ids, tok_state, cu_q, save_slot, runs)
+
+
+def hyper_mix_norm(xs, a=None, sa=1.0, b=None, sb=1.0, mix=None, outc=None, inc=None, w=None, eps=0.0, rows=None,
+                   out=None):
+    """Residual streams xs fp32 [T, S, d] (S <= 8).  With a sublayer output ``a`` (and ``b``): y = sa a + sb b, and all
+    streams at once xs[:, t] <- sum_s mix[s, t] xs[:, s] + outc[t] y.  With ``out``: the next sublayer's input
+    out[i] = rms_norm(sum_s inc[s] xs[rows[i], s]) * w from the same pass (inc None: the plain sum; rows None: row i;
+    rows only without an update)."""
+    if a is not None and rows is not None:
+        raise ValueError("hyper_mix_norm: gathered rows only without a stream update")
+    if _gpu(xs):
+        return _hyb().hyper_mix_norm(xs, a, float(sa), b, float(sb), mix, outc, inc, w, float(eps), rows, out)
+    return reference.hyper_mix_norm(xs, a, sa, b, sb, mix, outc, inc, w, eps, rows, out)
+
+
+def conv_qkv_cache(z, w, state, cu_q, row_seq, prev_row, runs, H, G, dk, dv, v_eps, slots, q_out, k_cache, v_cache,
+                   save_slot=None):
+    """z [T, H dk | G dk | G dv] (a view) through a causal per-channel convolution over every run of rows (w [C, taps],
+    no bias, y_t = sum_j w[:, j] z_(t - taps + 1 + j); inputs before a run from state[slot] [taps - 1, C] where
+    prev_row[first] <= -2, else zero); q -> q_out [T, H, dk]; k and v -- each value head brought to unit RMS (v_eps) --
+    into the token's rows of the paged caches (slot >= 0).  ``conv_state_update(z, state, ...)`` then stores the run's
+    newest inputs; where every row is a run of its own (cu_q None), ``save_slot`` makes this launch store them."""
+    if save_slot is not None and cu_q is not None:
+        raise ValueError("conv_qkv_cache: save_slot only where every row is a run of its own")
+    if _gpu(z):
+        return _hyb().conv_qkv_cache(z, w, state, cu_q, row_seq if cu_q is not None else None, prev_row, save_slot,
+                                     int(runs), int(H), int(G), int(dk), int(dv), float(v_eps), slots, q_out, k_cache,
+                                     v_cache)
+    reference.conv_qkv_cache(z, w, state, cu_q, prev_row, runs, H, G, dk, dv, v_eps, slots, q_out, k_cache, v_cache)
+    if save_slot is not None:
+        reference.conv_state_update(z, state, None, prev_row, save_slot, runs)
+
+
+def hyb_clamped_glu(gu, limit, alpha, out):
+    """``clamped_glu`` from the hybrid family's library (the same kernel)."""
+    if _gpu(gu):
+        return _hyb().clamped_glu(gu, float(limit), float(alpha), out)
+    return reference.clamped_glu(gu, limit, alpha, out)
+
+
+def logit_softcap(logits, cap):
+    """logits <- cap tanh(logits / cap), in place (fp32)."""
+    if _gpu(logits):
+        return _hyb().logit_softcap(logits, float(cap))
+    return reference.logit_softcap(logits, cap)

@@ -768,15 +768,21 @@ def rope_scaled_table(max_pos: int, dims: int, base: float, factor: float, origi
     return (torch.stack([torch.cos(a), torch.sin(a)], -1) * mag).float().to(device or "cpu")
 
 
-def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache) -> None:
+def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache, half_dims=0) -> None:
     T = z.shape[0]
     nq, nk, nv = H * dk, G * dk, G * dv
-    zf = z[:, :nq + nk + nv].float() + bias.float()[:nq + nk + nv]
-    cs = rope[positions[:T].long()][:, None]                  # [T, 1, rot / 2, 2]
-    rot = 2 * rope.shape[1]
+    zf = z[:, :nq + nk + nv].float()
+    if bias is not None:
+        zf = zf + bias.float()[:nq + nk + nv]
+    if rope is not None:
+        cs = rope[positions[:T].long()][:, None]                  # [T, 1, rot / 2, 2]
+        rot = 2 * rope.shape[1]
 
-    def turn(v):
-        return torch.cat([_rot_pairs(v[..., :rot], cs), v[..., rot:]], -1)
+        def turn(v):
+            return _rot_half(v, cs, half_dims) if half_dims else torch.cat([_rot_pairs(v[..., :rot], cs), v[..., rot:]], -1)
+    else:
+        def turn(v):
+            return v
 
     q_out.copy_(turn(zf[:, :nq].view(T, H, dk)).to(q_out.dtype))
     k = turn(zf[:, nq:nq + nk].view(T, G, dk)).to(k_cache.dtype)
@@ -787,7 +793,8 @@ def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache
     v_cache.view(-1, G, dv)[sl[keep]] = v[keep]
 
 
-def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias=None) -> None:
+def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, bias=None, keep_first=0,
+                sink=None) -> None:
     T, H, dk = q.shape
     BS, G = k_cache.shape[1], k_cache.shape[2]
     rep = H // G
@@ -795,7 +802,7 @@ def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, s
         p = int(positions[r])
         j0 = max(0, p - window + 1)
         bt = block_tables[int(row_seq[r])].long()
-        idx = torch.arange(j0, p + 1)
+        idx = torch.cat([torch.arange(0, min(keep_first, j0)), torch.arange(j0, p + 1)])
         K = k_cache[bt[idx // BS], idx % BS].float()            # [n, G, dk]
         V = v_cache[bt[idx // BS], idx % BS].float()
         qr = q[r].float().view(G, rep, dk)
@@ -803,6 +810,9 @@ def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, s
         if bias is not None:     # [2, H]: score -= bias[0, h] * ln(1 + bias[1, h] * distance)
             dist = (p - idx).float()
             s = s - (bias[0].float()[:, None] * torch.log1p(bias[1].float()[:, None] * dist[None, :])).view(G, rep, -1)
+        if sink is not None:     # one more logit in the denominator, without a value
+            s = torch.cat([s, sink.float().view(G, rep, 1)], -1)
+            V = torch.cat([V, torch.zeros_like(V[:1])], 0)
         o = torch.einsum("grn,ngv->grv", torch.softmax(s, -1), V).reshape(H, -1)
         if gate is not None:
             o = o * torch.sigmoid(gate[r].float())[:, None]
@@ -817,10 +827,13 @@ def _runs(T, cu_q, runs):
 
 
 def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
-               out) -> None:
+               out, mstate=None, mout=None) -> None:
     """S <- diag(a_t) S + b_t k_t v_t^T, o_t = S^T (q_scale q_t) (+ skip_h v_t) per head over every run of rows.
     mode 0: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel, b = 1;
-    mode 1: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) * b) per head.  q / k of head h: group h // hpg."""
+    mode 1: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) * b) per head.  q / k of head h: group h // hpg.
+    mode 2: log gates i = c tanh((dz[:, h] + dbias[h]) / c), f = logsigmoid(c tanh((dz[:, H + h] + dbias[H + h]) / c)),
+    c = dparam; running maximum m_t = max(f + m_(t-1), i) (carried in mstate, 0 at a sequence's start, written to mout);
+    a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); the state and the output have one more column, fed by v = 1."""
     T = q.shape[0]
     qf = q.float().reshape(T, -1, N) * q_scale
     kf, vf = k.float().reshape(T, -1, N), v.float().reshape(T, H, P)
@@ -828,9 +841,15 @@ def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, st
         ls = torch.nn.functional.logsigmoid(dz.float().reshape(T, H, N) + dbias.float().view(H, N))
         a = torch.exp(ls / float(dparam))                              # [T, H, N]
         b = torch.ones(T, H)
-    else:
+    elif mode == 1:
         b = torch.nn.functional.softplus(dz.float().reshape(T, H) + dbias.float(), beta=1.0, threshold=1e9)
         a = torch.exp(-torch.exp(dparam.float()) * b)[:, :, None].expand(T, H, N)
+    else:
+        c = float(dparam)
+        g = c * torch.tanh((dz.float().reshape(T, 2 * H) + dbias.float()) / c)
+        li, lf = g[:, :H], torch.nn.functional.logsigmoid(g[:, H:])
+        vf = torch.cat([vf, torch.ones(T, H, 1)], -1)
+        P = P + 1
     grp = torch.arange(H) // hpg
     o = out.view(T, H, P)
     for s0, s1 in _runs(T, cu_q, runs):
@@ -838,8 +857,17 @@ def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, st
             continue
         pr = int(prev_row[s0])
         S = state[-(pr + 2)].clone() if pr <= -2 else torch.zeros(H, N, P)
+        if mode == 2:
+            m = mstate[-(pr + 2)].clone() if pr <= -2 else torch.zeros(H)
         for t in range(s0, s1):
-            S = a[t][:, :, None] * S + (b[t][:, None] * kf[t, grp])[:, :, None] * vf[t][:, None, :]
+            if mode == 2:
+                mn = torch.maximum(lf[t] + m, li[t])
+                at, bt = torch.exp(lf[t] + m - mn)[:, None].expand(H, N), torch.exp(li[t] - mn)
+                m = mn
+                mout[t] = m
+            else:
+                at, bt = a[t], b[t]
+            S = at[:, :, None] * S + (bt[:, None] * kf[t, grp])[:, :, None] * vf[t][:, None, :]
             y = torch.einsum("hnp,hn->hp", S, qf[t, grp])
             if skip is not None:
                 y = y + skip.float()[:, None] * vf[t]
@@ -847,6 +875,17 @@ def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, st
         sv = int(save_slot[s1 - 1])
         if sv >= 0:
             state[sv] = S
+            if mode == 2:
+                mstate[sv] = m
+
+
+def memory_norm_gate(y, m, gate, w, eps, out) -> None:
+    """y [T, H, P + 1] (last column: the normaliser n . q), m [T, H]: o = y[..., :P] / (max(|n . q|, exp(-m)) + 1e-6),
+    brought to unit RMS per head, times w, times sigmoid(gate)."""
+    T, H, P1 = y.shape
+    den = torch.maximum(y[..., -1].abs(), torch.exp(-m)) + 1e-6
+    o = _unit_rms(y[..., :-1] / den[..., None], eps).reshape(T, H * (P1 - 1))
+    out.copy_((o * w.float() * torch.sigmoid(gate.float())).to(out.dtype))
 
 
 def gated_group_norm(y, gate, w, eps, group, gate_first, out) -> None:
@@ -898,12 +937,23 @@ def silu_mul(gate, up, out) -> None:
     out.copy_((g * torch.sigmoid(g) * up.float()).to(out.dtype))
 
 
-def softmax_topk(x, Wr, corr, k, ids, w) -> None:
+def softmax_topk(x, Wr, corr, k, ids, w, groups=1, keep=1, renorm=False) -> None:
     T = x.shape[0]
     s = torch.softmax(x.float() @ Wr.float().t(), -1)
-    pick = torch.argsort(s + corr.float(), dim=-1, descending=True, stable=True)[:, :k]
+    c = s + corr.float() if corr is not None else s
+    if keep < groups:            # only the experts of the ``keep`` groups with the largest best entry stay eligible
+        En = c.shape[1]
+        gs = c.view(T, groups, En // groups).max(-1).values
+        kept = torch.argsort(gs, dim=-1, descending=True, stable=True)[:, :keep]
+        ok = torch.zeros(T, groups, dtype=torch.bool)
+        ok.scatter_(1, kept, True)
+        c = torch.where(ok.repeat_interleave(En // groups, 1), c, torch.full_like(c, -float("inf")))
+    pick = torch.argsort(c, dim=-1, descending=True, stable=True)[:, :k]
+    wt = torch.gather(s, 1, pick)
+    if renorm:
+        wt = wt / (wt.sum(-1, keepdim=True) + 1e-20)
     ids[: T * k].copy_(pick.reshape(-1).int())
-    w[: T * k].copy_(torch.gather(s, 1, pick).reshape(-1))
+    w[: T * k].copy_(wt.reshape(-1))
 
 
 def moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out) -> None:
@@ -966,3 +1016,70 @@ def gelu_tanh_mul(gate, up, out) -> None:
 
 def sigmoid_mul(a, gate, out) -> None:
     out.copy_((a.float() * torch.sigmoid(gate.float())).to(out.dtype))
+
+
+# ---- several residual streams, hashed token pairs, convolved projections (the Dalalix layers) -------------------
+def embed_pair_hash(ids, table, pair_table, buckets, mul_prev, mul_cur, prev_row, tok_state, x) -> None:
+    """x [T, S, d]: every stream = table[token] + pair_table[(prev * mul_prev + token * mul_cur) mod buckets]; a row
+    without a previous token takes pair_table[buckets]."""
+    T = x.shape[0]
+    tok = ids[:T].long()
+    e = table[tok].float()
+    if pair_table is not None:
+        pr = prev_row[:T].long()
+        prev = torch.where(pr >= 0, tok[pr.clamp(min=0)], tok_state[(-(pr + 2)).clamp(min=0)].long())
+        rows = torch.where(pr == -1, torch.full_like(tok, buckets), (prev * mul_prev + tok * mul_cur) % buckets)
+        e = e + pair_table[rows].float()
+    x.copy_(e[:, None, :].expand_as(x))
+
+
+def token_state_update(ids, tok_state, cu_q, save_slot, runs) -> None:
+    T = ids.shape[0]
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 > s0 and int(save_slot[s1 - 1]) >= 0:
+            tok_state[int(save_slot[s1 - 1])] = ids[s1 - 1]
+
+
+def hyper_mix_norm(xs, a, sa, b, sb, mix, outc, inc, w, eps, rows, out) -> None:
+    """xs [T, S, d] fp32.  With ``a``: y = sa a + sb b; xs[:, t] <- sum_s mix[s, t] xs[:, s] + outc[t] y.  Then
+    out[i] = rms_norm(sum_s inc[s] xs[rows[i], s]) * w (inc None: the plain sum)."""
+    if a is not None:
+        y = sa * a.float()
+        if b is not None:
+            y = y + sb * b.float()
+        xs.copy_(torch.einsum("st,nsd->ntd", mix.float(), xs)
+                 + outc.float()[None, :, None] * y[:, None, :])
+    if out is not None:
+        src = xs if rows is None else xs[rows.long()]
+        n = out.shape[0]
+        u = src[:n].sum(1) if inc is None else torch.einsum("s,nsd->nd", inc.float(), src[:n])
+        out.copy_((_unit_rms(u, eps) * w.float()).to(out.dtype))
+
+
+def conv_qkv_cache(z, w, state, cu_q, prev_row, runs, H, G, dk, dv, v_eps, slots, q_out, k_cache, v_cache) -> None:
+    """z [T, H dk | G dk | G dv] through a causal per-channel convolution (w [C, taps], no bias, inputs before a run
+    from state [slots, taps - 1, C]); q -> q_out, k and the unit-RMS (per head, v_eps) v -> the paged caches."""
+    T = z.shape[0]
+    C, taps = w.shape
+    nq, nk = H * dk, G * dk
+    y = torch.zeros(T, C)
+    zf, wf = z.float(), w.float()
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 <= s0:
+            continue
+        pr = int(prev_row[s0])
+        hist = state[-(pr + 2)].float() if pr <= -2 else torch.zeros(taps - 1, C)
+        full = torch.cat([hist, zf[s0:s1]], 0)
+        for j in range(taps):
+            y[s0:s1] += full[j:j + s1 - s0] * wf[:, j]
+    q_out.copy_(y[:, :nq].view(T, H, dk).to(q_out.dtype))
+    k = y[:, nq:nq + nk].view(T, G, dk).to(k_cache.dtype)
+    v = _unit_rms(y[:, nq + nk:].view(T, G, dv), v_eps).to(v_cache.dtype)
+    sl = slots[:T].long()
+    keep = sl >= 0
+    k_cache.view(-1, G, dk)[sl[keep]] = k[keep]
+    v_cache.view(-1, G, dv)[sl[keep]] = v[keep]
+
+
+def logit_softcap(logits, cap) -> None:
+    logits.copy_(cap * torch.tanh(logits / cap))
