@@ -1,4 +1,4 @@
-// TORCH_LIBRARY registration of the kernels in hybrid_rows.hip, window_attention.hip and decay_scan.hip, plus the
+// TORCH_LIBRARY registration of the kernels in hybrid_rows.hip, stream_rows.hip, window_attention.hip and decay_scan.hip, plus the
 // expert-segment kernels of glu_moe.hip that the routed feed-forward shares (symmetry_amd/_C_hybrid.so, namespace
 // symmetry_amd_hybrid).
 //
@@ -140,9 +140,9 @@ void residual_mix_norm(Tensor& x, const Tensor& a, double sa, const OptTensor& b
   launch_residual_mix_norm(r, f32, cur_stream(x));
 }
 
-void qkv_rope_cache(const Tensor& z, const Tensor& bias, int64_t H, int64_t G, int64_t dk, int64_t dv,
-                    const Tensor& positions, const Tensor& slots, const Tensor& rope, Tensor& q_out, Tensor& k_cache,
-                    Tensor& v_cache) {
+void qkv_rope_cache(const Tensor& z, const OptTensor& bias, int64_t H, int64_t G, int64_t dk, int64_t dv,
+                    const Tensor& positions, const Tensor& slots, const OptTensor& rope, Tensor& q_out, Tensor& k_cache,
+                    Tensor& v_cache, int64_t half_dims) {
   const int f32 = act(z, "z", false);
   TORCH_CHECK(z.dim() == 2, "qkv_rope_cache: z [T, n]");
   const int64_t T = z.size(0), n = H * dk + G * dk + G * dv;
@@ -152,21 +152,29 @@ void qkv_rope_cache(const Tensor& z, const Tensor& bias, int64_t H, int64_t G, i
   same_act(q_out, f32, "q_out");
   same_act(k_cache, f32, "k_cache");
   same_act(v_cache, f32, "v_cache");
-  dtype(bias, at::kFloat, "bias");
   dtype(positions, at::kInt, "positions");
   dtype(slots, at::kInt, "slots");
-  dtype(rope, at::kFloat, "rope");
-  TORCH_CHECK(rope.dim() == 3 && rope.size(2) == 2 && 2 * rope.size(1) <= dk, "qkv_rope_cache: rope [max_pos, pairs, 2]");
-  TORCH_CHECK(bias.numel() >= n && q_out.numel() == T * H * dk && positions.numel() >= T && slots.numel() >= T &&
+  if (bias.has_value()) {
+    dtype(*bias, at::kFloat, "bias");
+    TORCH_CHECK(bias->numel() >= n, "qkv_rope_cache: bias shorter than q | k | v");
+  }
+  if (rope.has_value()) {
+    dtype(*rope, at::kFloat, "rope");
+    TORCH_CHECK(rope->dim() == 3 && rope->size(2) == 2 && 2 * rope->size(1) <= dk,
+                "qkv_rope_cache: rope [max_pos, pairs, 2]");
+    TORCH_CHECK(half_dims == 0 || half_dims == 2 * rope->size(1), "qkv_rope_cache: half_dims = 2 * pairs of the table");
+  }
+  TORCH_CHECK(q_out.numel() == T * H * dk && positions.numel() >= T && slots.numel() >= T &&
                   k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(2) == G && k_cache.size(3) == dk &&
                   v_cache.size(2) == G && v_cache.size(3) == dv && H % G == 0,
               "qkv_rope_cache: shapes");
   a.z = z.data_ptr();
-  a.bias = ptr<float>(bias);
-  a.H = (int)H, a.G = (int)G, a.dk = (int)dk, a.dv = (int)dv, a.pairs = (int)rope.size(1);
+  a.bias = optptr<float>(bias);
+  a.H = (int)H, a.G = (int)G, a.dk = (int)dk, a.dv = (int)dv, a.pairs = rope.has_value() ? (int)rope->size(1) : 0;
+  a.half = half_dims > 0;
   a.positions = ptr<int>(positions);
   a.slots = ptr<int>(slots);
-  a.rope = ptr<float>(rope);
+  a.rope = optptr<float>(rope);
   a.q_out = q_out.data_ptr();
   a.k_cache = k_cache.data_ptr();
   a.v_cache = v_cache.data_ptr();
@@ -175,7 +183,8 @@ void qkv_rope_cache(const Tensor& z, const Tensor& bias, int64_t H, int64_t G, i
 
 int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_tables,
                     const Tensor& row_seq, const Tensor& positions, int64_t window, double scale, const OptTensor& gate,
-                    Tensor& out, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl, const OptTensor& bias) {
+                    Tensor& out, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl, const OptTensor& bias,
+                    int64_t keep_first, const OptTensor& sink) {
   const int f32 = act(q, "q");
   same_act(k_cache, f32, "k_cache");
   same_act(v_cache, f32, "v_cache");
@@ -202,6 +211,13 @@ int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cach
     TORCH_CHECK(bias->dim() == 2 && bias->size(0) == 2 && bias->size(1) == a.H, "window_attn: bias [2, H]");
     a.bias = ptr<float>(*bias);
   }
+  if (sink.has_value()) {
+    dtype(*sink, at::kFloat, "sink");
+    TORCH_CHECK(sink->numel() == a.H, "window_attn: sink [H]");
+    a.sink = ptr<float>(*sink);
+  }
+  TORCH_CHECK(keep_first >= 0 && keep_first < (1LL << 30), "window_attn: keep_first");
+  a.keep_first = (int)keep_first;
   if (tiles.has_value() && cu_q.has_value()) {
     dtype(*tiles, at::kInt, "tiles");
     dtype(*cu_q, at::kInt, "cu_q");
@@ -224,25 +240,33 @@ int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cach
 void decay_scan(int64_t mode, const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& dz, const Tensor& dbias,
                 const OptTensor& rate, double tau, const OptTensor& skip, double q_scale, int64_t H, int64_t N, int64_t P,
                 int64_t hpg, Tensor& state, const OptTensor& cu_q, const Tensor& prev_row, const Tensor& save_slot,
-                int64_t runs, Tensor& out) {
+                int64_t runs, Tensor& out, const OptTensor& mout) {
   const int f32 = act(v, "v", false);
   dtype(out, at::kFloat, "out");
   dtype(dbias, at::kFloat, "dbias");
   dtype(prev_row, at::kInt, "prev_row");
   dtype(save_slot, at::kInt, "save_slot");
   gpu(state, "state");
-  TORCH_CHECK(mode == 0 || mode == 1, "decay_scan: mode");
-  TORCH_CHECK(state.scalar_type() == at::kFloat && state.dim() == 4 && state.size(1) == H && state.size(2) == N &&
-                  state.size(3) == P, "decay_scan: state [slots, H, N, P] fp32");
+  TORCH_CHECK(mode >= 0 && mode <= 2, "decay_scan: mode");
+  const int64_t PS = mode == 2 ? P + 1 : P;      // columns of the state and of out
+  TORCH_CHECK(state.scalar_type() == at::kFloat && state.dim() == 4 && state.size(1) == H &&
+                  state.size(2) == (mode == 2 ? N + 1 : N) && state.size(3) == PS,
+              "decay_scan: state [slots, H, N, P] fp32 (log gates: [slots, H, N + 1, P + 1])");
   TORCH_CHECK(H > 0 && hpg > 0 && H % hpg == 0 && N >= 1 && N <= 256 && P >= 1 && runs <= 65535, "decay_scan: sizes");
   const int64_t T = v.size(0), groups = H / hpg;
   DecayScanArgs a{};
   a.ldq = view2(q, f32, T, groups * N, "q");
   a.ldk = view2(k, f32, T, groups * N, "k");
   a.ldv = view2(v, f32, T, H * P, "v");
-  a.ldd = view2(dz, f32, T, mode == 0 ? H * N : H, "dz");
-  TORCH_CHECK(dbias.numel() == (mode == 0 ? H * N : H) && out.numel() == T * H * P && prev_row.numel() >= T &&
-                  save_slot.numel() >= T, "decay_scan: shapes");
+  a.ldd = view2(dz, mode == 2 ? 1 : f32, T, mode == 0 ? H * N : (mode == 1 ? H : 2 * H), "dz");
+  TORCH_CHECK(dbias.numel() == (mode == 0 ? H * N : (mode == 1 ? H : 2 * H)) && out.numel() == T * H * PS &&
+                  prev_row.numel() >= T && save_slot.numel() >= T, "decay_scan: shapes");
+  if (mode == 2) {
+    TORCH_CHECK(mout.has_value() && !skip.has_value(), "decay_scan: the log-gate mode writes its maxima and has no skip");
+    dtype(*mout, at::kFloat, "mout");
+    TORCH_CHECK(mout->numel() == T * H, "decay_scan: mout [T, H]");
+    a.mout = ptr<float>(*mout);
+  }
   if (mode == 1) {
     TORCH_CHECK(rate.has_value(), "decay_scan: the step-size mode needs the per-head rates");
     dtype(*rate, at::kFloat, "rate");
@@ -268,7 +292,7 @@ void decay_scan(int64_t mode, const Tensor& q, const Tensor& k, const Tensor& v,
   a.dbias = ptr<float>(dbias);
   a.tau = (float)tau;
   a.q_scale = (float)q_scale;
-  a.H = (int)H, a.N = (int)N, a.P = (int)P, a.hpg = (int)hpg;
+  a.H = (int)H, a.N = (int)N, a.P = (int)PS, a.vcols = (int)P, a.hpg = (int)hpg;
   a.state = ptr<float>(state);
   a.state_stride = state.stride(0);
   a.prev_row = ptr<int>(prev_row);
@@ -372,18 +396,21 @@ void silu_mul(const Tensor& gate, const Tensor& up, Tensor& out) {
                   cur_stream(out));
 }
 
-void softmax_topk(const Tensor& x, const Tensor& Wr, const Tensor& corr, int64_t k, Tensor& ids, Tensor& w) {
+void softmax_topk(const Tensor& x, const Tensor& Wr, const OptTensor& corr, int64_t k, Tensor& ids, Tensor& w,
+                  int64_t groups, int64_t keep, bool renorm) {
   const int f32 = act(x, "x");
   same_act(Wr, f32, "Wr");
-  dtype(corr, at::kFloat, "corr");
+  if (corr.has_value()) dtype(*corr, at::kFloat, "corr");
   dtype(ids, at::kInt, "ids");
   dtype(w, at::kFloat, "w");
   TORCH_CHECK(x.dim() == 2 && Wr.dim() == 2, "softmax_topk: x [T, d], Wr [En, d]");
   const int64_t T = x.size(0), d = x.size(1), En = Wr.size(0);
-  TORCH_CHECK(Wr.size(1) == d && corr.numel() == En && k >= 1 && k <= En && En <= 4096 && ids.numel() >= T * k &&
-                  w.numel() >= T * k, "softmax_topk: shapes");
-  launch_softmax_topk(x.data_ptr(), Wr.data_ptr(), ptr<float>(corr), (int)T, (int)d, (int)En, (int)k, ptr<int>(ids),
-                      ptr<float>(w), f32, cur_stream(x));
+  TORCH_CHECK(Wr.size(1) == d && (!corr.has_value() || corr->numel() == En) && k >= 1 && k <= En && En <= 4096 &&
+                  ids.numel() >= T * k && w.numel() >= T * k, "softmax_topk: shapes");
+  TORCH_CHECK(groups >= 1 && groups <= 64 && En % groups == 0 && keep >= 1 && keep <= groups && k <= keep * (En / groups),
+              "softmax_topk: groups (at most 64, equal sizes) / keep / k");
+  launch_softmax_topk(x.data_ptr(), Wr.data_ptr(), optptr<float>(corr), (int)T, (int)d, (int)En, (int)k, (int)groups,
+                      (int)keep, renorm ? 1 : 0, ptr<int>(ids), ptr<float>(w), f32, cur_stream(x));
 }
 
 void moe_mix(const Tensor& y, const Tensor& dst, const Tensor& ids, const Tensor& w, int64_t k, int64_t E, const Tensor& h,
@@ -568,6 +595,185 @@ void sigmoid_mul(const Tensor& a, const Tensor& gate, Tensor& out) {
                      cur_stream(out));
 }
 
+
+// ---- several residual streams, hashed token pairs, convolved projections, the matrix memory's read-out ------------
+void embed_pair_hash(const Tensor& ids, const OptTensor& src, const OptTensor& prev, const Tensor& table,
+                     const OptTensor& pair_table, int64_t buckets, int64_t mul_prev, int64_t mul_cur, const Tensor& prev_row,
+                     Tensor& tok_state, const OptTensor& save_slot, Tensor& x) {
+  const int f32 = act(table, "table");
+  dtype(ids, at::kInt, "ids");
+  dtype(x, at::kFloat, "x");
+  dtype(prev_row, at::kInt, "prev_row");
+  dtype(tok_state, at::kInt, "tok_state");
+  TORCH_CHECK(x.dim() == 3 && table.dim() == 2 && x.size(2) == table.size(1), "embed_pair_hash: x [T, S, d], table [V, d]");
+  const int64_t T = x.size(0), S = x.size(1), d = x.size(2);
+  TORCH_CHECK(ids.numel() >= T && prev_row.numel() >= T && S >= 1 && S <= 8, "embed_pair_hash: shapes (at most 8 streams)");
+  PairHashArgs a{};
+  if (src.has_value()) {
+    TORCH_CHECK(prev.has_value(), "embed_pair_hash: src without prev");
+    dtype(*src, at::kInt, "src");
+    dtype(*prev, at::kInt, "prev");
+    TORCH_CHECK(src->numel() >= T, "embed_pair_hash: src too short");
+    a.src = ptr<int>(*src), a.prev = ptr<int>(*prev);
+  }
+  if (pair_table.has_value()) {
+    same_act(*pair_table, f32, "pair_table");
+    TORCH_CHECK(pair_table->dim() == 2 && pair_table->size(0) == buckets + 1 && pair_table->size(1) == d && buckets >= 1,
+                "embed_pair_hash: pair_table [buckets + 1, d]");
+    a.pair_table = pair_table->data_ptr();
+  }
+  if (save_slot.has_value()) {
+    dtype(*save_slot, at::kInt, "save_slot");
+    TORCH_CHECK(save_slot->numel() >= T, "embed_pair_hash: save_slot too short");
+    a.save_slot = ptr<int>(*save_slot);
+  }
+  a.ids = ptr<int>(ids);
+  a.table = table.data_ptr();
+  a.buckets = buckets, a.mul_prev = mul_prev, a.mul_cur = mul_cur;
+  a.prev_row = ptr<int>(prev_row);
+  a.tok_state = ptr<int>(tok_state);
+  a.x = ptr<float>(x);
+  a.T = (int)T, a.S = (int)S, a.d = (int)d;
+  launch_embed_pair_hash(a, f32, cur_stream(x));
+}
+
+void token_state_update(const Tensor& ids, Tensor& tok_state, const OptTensor& cu_q, const Tensor& save_slot, int64_t runs) {
+  dtype(ids, at::kInt, "ids");
+  dtype(tok_state, at::kInt, "tok_state");
+  dtype(save_slot, at::kInt, "save_slot");
+  if (cu_q.has_value()) {
+    dtype(*cu_q, at::kInt, "cu_q");
+    TORCH_CHECK(cu_q->numel() >= runs + 1, "token_state_update: cu_q too short");
+  } else {
+    TORCH_CHECK(runs <= ids.numel(), "token_state_update: more runs than rows");
+  }
+  launch_token_state_update(ptr<int>(ids), ptr<int>(tok_state), optptr<int>(cu_q), ptr<int>(save_slot), (int)runs,
+                            cur_stream(ids));
+}
+
+void hyper_mix_norm(Tensor& xs, const OptTensor& a_, double sa, const OptTensor& b_, double sb, const OptTensor& mix,
+                    const OptTensor& outc, const OptTensor& inc, const OptTensor& w, double eps, const OptTensor& rows,
+                    const OptTensor& out) {
+  dtype(xs, at::kFloat, "xs");
+  TORCH_CHECK(xs.dim() == 3, "hyper_mix_norm: xs [T, S, d]");
+  const int64_t T = xs.size(0), S = xs.size(1), d = xs.size(2);
+  TORCH_CHECK(S >= 1 && S <= 8 && d >= 1 && d <= 15000, "hyper_mix_norm: at most 8 streams, width at most 15000");
+  HyperMixArgs a{};
+  a.xs = ptr<float>(xs);
+  a.T = (int)T, a.S = (int)S, a.d = (int)d;
+  if (a_.has_value()) {
+    a.a_f32 = act(*a_, "a");
+    TORCH_CHECK(a_->numel() == T * d && mix.has_value() && outc.has_value() && !rows.has_value(),
+                "hyper_mix_norm: a [T, d] with mix and outc, no gathered rows");
+    dtype(*mix, at::kFloat, "mix");
+    dtype(*outc, at::kFloat, "outc");
+    TORCH_CHECK(mix->numel() == S * S && outc->numel() == S, "hyper_mix_norm: mix [S, S], outc [S]");
+    a.a = a_->data_ptr(), a.sa = (float)sa, a.mix = ptr<float>(*mix), a.outc = ptr<float>(*outc);
+    if (b_.has_value()) {
+      a.b_f32 = act(*b_, "b");
+      TORCH_CHECK(b_->numel() == T * d, "hyper_mix_norm: b [T, d]");
+      a.b = b_->data_ptr(), a.sb = (float)sb;
+    }
+  }
+  int f32 = 0;
+  if (out.has_value()) {
+    f32 = act(*out, "out");
+    TORCH_CHECK(out->dim() == 2 && out->size(1) == d && w.has_value(), "hyper_mix_norm: out [n, d] with w");
+    dtype(*w, at::kFloat, "w");
+    TORCH_CHECK(w->numel() == d, "hyper_mix_norm: w [d]");
+    a.n = (int)out->size(0);
+    if (rows.has_value()) {
+      dtype(*rows, at::kLong, "rows");
+      TORCH_CHECK(rows->numel() >= a.n, "hyper_mix_norm: rows too short");
+      a.rows = reinterpret_cast<const long long*>(rows->data_ptr());
+    } else {
+      TORCH_CHECK(a.n <= T, "hyper_mix_norm: more output rows than rows");
+    }
+    if (inc.has_value()) {
+      dtype(*inc, at::kFloat, "inc");
+      TORCH_CHECK(inc->numel() == S, "hyper_mix_norm: inc [S]");
+      a.inc = ptr<float>(*inc);
+    }
+    a.w = ptr<float>(*w), a.eps = (float)eps, a.out = out->data_ptr();
+  }
+  TORCH_CHECK(T <= 65535 * 1024 && a.n <= 65535 * 1024, "hyper_mix_norm: too many rows");
+  launch_hyper_mix_norm(a, f32, cur_stream(xs));
+}
+
+void conv_qkv_cache(const Tensor& z, const Tensor& w, Tensor& state, const OptTensor& cu_q, const OptTensor& row_seq,
+                    const Tensor& prev_row, const OptTensor& save_slot, int64_t runs, int64_t H, int64_t G, int64_t dk,
+                    int64_t dv, double v_eps, const Tensor& slots, Tensor& q_out, Tensor& k_cache, Tensor& v_cache) {
+  const int f32 = act(z, "z", false);
+  TORCH_CHECK(z.dim() == 2 && state.dim() == 3 && w.dim() == 2, "conv_qkv_cache: z [T, C], w [C, taps], state [slots, taps - 1, C]");
+  const int64_t T = z.size(0), C = H * dk + G * dk + G * dv;
+  ConvQkvArgs a{};
+  a.ldz = view2(z, f32, T, C, "z");
+  same_act(w, f32, "w");
+  same_act(state, f32, "state");
+  same_act(q_out, f32, "q_out");
+  same_act(k_cache, f32, "k_cache");
+  same_act(v_cache, f32, "v_cache");
+  dtype(prev_row, at::kInt, "prev_row");
+  dtype(slots, at::kInt, "slots");
+  const int64_t taps = w.size(1);
+  TORCH_CHECK(w.size(0) == C && taps >= 1 && taps <= 16 && state.size(1) == taps - 1 && state.size(2) == C && C <= 15000 &&
+                  H % G == 0 && q_out.numel() == T * H * dk && prev_row.numel() >= T && slots.numel() >= T &&
+                  k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(2) == G && k_cache.size(3) == dk &&
+                  v_cache.size(2) == G && v_cache.size(3) == dv && T <= 65535 * 1024,
+              "conv_qkv_cache: shapes (at most 16 taps, 15000 channels)");
+  if (cu_q.has_value()) {
+    TORCH_CHECK(row_seq.has_value(), "conv_qkv_cache: cu_q without row_seq");
+    dtype(*cu_q, at::kInt, "cu_q");
+    dtype(*row_seq, at::kInt, "row_seq");
+    TORCH_CHECK(cu_q->numel() >= runs + 1 && row_seq->numel() >= T, "conv_qkv_cache: cu_q / row_seq too short");
+    a.cu_q = ptr<int>(*cu_q), a.row_seq = ptr<int>(*row_seq);
+  } else {
+    TORCH_CHECK(runs <= T, "conv_qkv_cache: more runs than rows");
+  }
+  if (save_slot.has_value()) {
+    TORCH_CHECK(!cu_q.has_value(), "conv_qkv_cache: save_slot only where every row is a run of its own");
+    dtype(*save_slot, at::kInt, "save_slot");
+    TORCH_CHECK(save_slot->numel() >= T, "conv_qkv_cache: save_slot too short");
+    a.save_slot = ptr<int>(*save_slot);
+  }
+  a.z = z.data_ptr(), a.w = w.data_ptr(), a.state = state.data_ptr();
+  a.state_stride = state.stride(0);
+  a.prev_row = ptr<int>(prev_row), a.slots = ptr<int>(slots);
+  a.q_out = q_out.data_ptr(), a.k_cache = k_cache.data_ptr(), a.v_cache = v_cache.data_ptr();
+  a.v_eps = (float)v_eps;
+  a.T = (int)T, a.C = (int)C, a.taps = (int)taps, a.H = (int)H, a.G = (int)G, a.dk = (int)dk, a.dv = (int)dv;
+  launch_conv_qkv_cache(a, f32, cur_stream(z));
+}
+
+void memory_norm_gate(const Tensor& y, const Tensor& m, const Tensor& gate, const Tensor& w, double eps, Tensor& out) {
+  const int f32 = act(out, "out");
+  dtype(y, at::kFloat, "y");
+  dtype(m, at::kFloat, "m");
+  dtype(w, at::kFloat, "w");
+  TORCH_CHECK(y.dim() == 3 && y.size(2) >= 2, "memory_norm_gate: y [T, H, P + 1]");
+  const int64_t T = y.size(0), H = y.size(1), P = y.size(2) - 1;
+  const int64_t ldg = view2(gate, f32, T, H * P, "gate");
+  TORCH_CHECK(m.numel() == T * H && w.numel() == H * P && out.numel() == T * H * P && H <= 65535 && T <= 65535 * 1024,
+              "memory_norm_gate: shapes");
+  launch_memory_norm_gate(ptr<float>(y), ptr<float>(m), gate.data_ptr(), ldg, ptr<float>(w), (float)eps, out.data_ptr(),
+                          (int)T, (int)H, (int)P, f32, cur_stream(y));
+}
+
+void hyb_clamped_glu(const Tensor& gu, double limit, double alpha, Tensor& out) {
+  const int f32 = act(gu, "gu");
+  same_act(out, f32, "out");
+  TORCH_CHECK(gu.dim() == 2 && out.dim() == 2 && gu.size(0) == out.size(0) && gu.size(1) == 2 * out.size(1),
+              "clamped_glu: gu [R, 2F], out [R, F]");
+  launch_clamped_glu(gu.data_ptr(), out.data_ptr(), (int)out.size(0), (int)out.size(1), (float)limit, (float)alpha, f32,
+                     cur_stream(gu));
+}
+
+void logit_softcap(Tensor& logits, double cap) {
+  dtype(logits, at::kFloat, "logits");
+  TORCH_CHECK(cap > 0, "logit_softcap: cap");
+  launch_logit_softcap(ptr<float>(logits), logits.numel(), (float)cap, cur_stream(logits));
+}
+
 }  // namespace
 
 TORCH_LIBRARY(symmetry_amd_hybrid, m) {
@@ -579,17 +785,18 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
       "Tensor? w, float eps, float offset, Tensor(b!)? out) -> ()",
       &residual_mix_norm);
   m.def(
-      "qkv_rope_cache(Tensor z, Tensor bias, int H, int G, int dk, int dv, Tensor positions, Tensor slots, Tensor rope, "
-      "Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()",
+      "qkv_rope_cache(Tensor z, Tensor? bias, int H, int G, int dk, int dv, Tensor positions, Tensor slots, Tensor? rope, "
+      "Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache, int half_dims) -> ()",
       &qkv_rope_cache);
   m.def(
       "window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor row_seq, Tensor positions, "
-      "int window, float scale, Tensor? gate, Tensor(a!) out, Tensor? tiles, Tensor? cu_q, int impl, Tensor? bias) -> int",
+      "int window, float scale, Tensor? gate, Tensor(a!) out, Tensor? tiles, Tensor? cu_q, int impl, Tensor? bias, "
+      "int keep_first, Tensor? sink) -> int",
       &window_attn);
   m.def(
       "decay_scan(int mode, Tensor q, Tensor k, Tensor v, Tensor dz, Tensor dbias, Tensor? rate, float tau, Tensor? skip, "
       "float q_scale, int H, int N, int P, int hpg, Tensor(a!) state, Tensor? cu_q, Tensor prev_row, Tensor save_slot, "
-      "int runs, Tensor(b!) out) -> ()",
+      "int runs, Tensor(b!) out, Tensor(c!)? mout) -> ()",
       &decay_scan);
   m.def("gated_group_norm(Tensor y, Tensor gate, Tensor w, float eps, int group, bool gate_first, Tensor(a!) out) -> ()",
         &gated_group_norm);
@@ -601,7 +808,10 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
         &conv_state_update);
   m.def("relu_sq(Tensor a, Tensor(a!) out) -> ()", &relu_sq);
   m.def("silu_mul(Tensor gate, Tensor up, Tensor(a!) out) -> ()", &silu_mul);
-  m.def("softmax_topk(Tensor x, Tensor Wr, Tensor corr, int k, Tensor(a!) ids, Tensor(b!) w) -> ()", &softmax_topk);
+  m.def(
+      "softmax_topk(Tensor x, Tensor Wr, Tensor? corr, int k, Tensor(a!) ids, Tensor(b!) w, int groups, int keep, "
+      "bool renorm) -> ()",
+      &softmax_topk);
   m.def(
       "moe_mix(Tensor y, Tensor dst, Tensor ids, Tensor w, int k, int E, Tensor h, Tensor? shared, Tensor? sgate, "
       "Tensor(a!) out) -> ()",
@@ -628,4 +838,22 @@ TORCH_LIBRARY(symmetry_amd_hybrid, m) {
       &qk_norm_cache);
   m.def("gelu_tanh_mul(Tensor gate, Tensor up, Tensor(a!) out) -> ()", &gelu_tanh_mul);
   m.def("sigmoid_mul(Tensor a, Tensor gate, Tensor(a!) out) -> ()", &sigmoid_mul);
+  m.def(
+      "embed_pair_hash(Tensor ids, Tensor? src, Tensor? prev, Tensor table, Tensor? pair_table, int buckets, int mul_prev, "
+      "int mul_cur, Tensor prev_row, Tensor(a!) tok_state, Tensor? save_slot, Tensor(b!) x) -> ()",
+      &embed_pair_hash);
+  m.def("token_state_update(Tensor ids, Tensor(a!) tok_state, Tensor? cu_q, Tensor save_slot, int runs) -> ()",
+        &token_state_update);
+  m.def(
+      "hyper_mix_norm(Tensor(a!) xs, Tensor? a, float sa, Tensor? b, float sb, Tensor? mix, Tensor? outc, Tensor? inc, "
+      "Tensor? w, float eps, Tensor? rows, Tensor(b!)? out) -> ()",
+      &hyper_mix_norm);
+  m.def(
+      "conv_qkv_cache(Tensor z, Tensor w, Tensor(a!) state, Tensor? cu_q, Tensor? row_seq, Tensor prev_row, "
+      "Tensor? save_slot, int runs, int H, int G, int dk, int dv, float v_eps, Tensor slots, Tensor(b!) q_out, "
+      "Tensor(c!) k_cache, Tensor(d!) v_cache) -> ()",
+      &conv_qkv_cache);
+  m.def("memory_norm_gate(Tensor y, Tensor m, Tensor gate, Tensor w, float eps, Tensor(a!) out) -> ()", &memory_norm_gate);
+  m.def("clamped_glu(Tensor gu, float limit, float alpha, Tensor(a!) out) -> ()", &hyb_clamped_glu);
+  m.def("logit_softcap(Tensor(a!) logits, float cap) -> ()", &logit_softcap);
 }

@@ -5,6 +5,12 @@
 //
 // mode 0 (channel gate): a_t[n] = sigmoid(dz_t[n] + dbias[n])^(1 / tau) = exp(logsigmoid(.) / tau), b_t = 1
 // mode 1 (step size):    b_t = softplus(dz_t + dbias[h]), a_t = exp(-exp(rate[h]) b_t) for every n
+// mode 2 (log gates):    i_t = c tanh(. / c), f_t = logsigmoid(c tanh(. / c)) from fp32 pre-activations, a running maximum
+//                        m_t = max(f_t + m_(t-1), i_t) (m = 0 at a sequence's start), a_t = exp(f_t + m_(t-1) - m_t),
+//                        b_t = exp(i_t - m_t).  One more value column is fed by v = 1: its state is the normaliser n_t and
+//                        its output n_t . q_t.  m travels in one more row of the state, the same value in every column, so
+//                        that each column's owner reads and writes its own copy (no workgroup reads what another writes);
+//                        it is chained token by token by the first wave while a batch is staged.
 //
 // The state walks token by token in fp32, in the same order however a prompt is cut into steps, so a position's
 // output does not depend on the cut.  A run of rows (one sequence's tokens of this step) starts from its state slot
@@ -36,7 +42,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   constexpr int LROW = SLICES * (NPL + 4);                  // a token's LDS row: the four slices 16 bytes apart in bank
                                                             // space, so the lanes' four addresses of a read do not collide
   constexpr int EPT = CH * NPAD / NT;                       // staged (token, channel) entries per thread
-  constexpr int ASZ = MODE == 0 ? CH * LROW : 2 * CH;       // decays per channel, or (decay, step) per token
+  constexpr int ASZ = MODE == 0 ? CH * LROW : (MODE == 1 ? 2 : 3) * CH;   // decays per channel, or (decay, step(, max)) per token
   constexpr int BUF = 2 * CH * LROW + ASZ;
   static_assert(CH * NPAD % NT == 0, "staging split");
   const int N = a.N, P = a.P;
@@ -54,23 +60,29 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   const int sv = a.save_slot[s1 - 1];
   float S[NPL];
   if (pr <= -2 && pin) {
-    const float* st = a.state + (long long)(-(pr + 2)) * a.state_stride + (long long)h * N * P + p;
+    const float* st = a.state + (long long)(-(pr + 2)) * a.state_stride + (long long)h * (N + (MODE == 2)) * P + p;
 #pragma unroll
     for (int i = 0; i < NPL; ++i) S[i] = n0 + i < N ? st[(long long)(n0 + i) * P] : 0.f;
   } else {
 #pragma unroll
     for (int i = 0; i < NPL; ++i) S[i] = 0.f;
   }
+  // mode 2: the running maximum, chained by the first wave (every lane of it holds the same value); a workgroup reads
+  // the copy in its first column (every workgroup has one)
+  float mrun = 0.f;
+  if (MODE == 2 && pr <= -2)
+    mrun = a.state[(long long)(-(pr + 2)) * a.state_stride + ((long long)h * (N + 1) + N) * P + blockIdx.x * (PCOLS * (NT / 64))];
   const T* q = reinterpret_cast<const T*>(a.q) + (long long)grp * N;
   const T* k = reinterpret_cast<const T*>(a.k) + (long long)grp * N;
-  const T* v = reinterpret_cast<const T*>(a.v) + (long long)h * P + p;
+  const T* v = reinterpret_cast<const T*>(a.v) + (long long)h * a.vcols + p;
+  const bool vin = p < a.vcols;        // (mode 2: column vcols is fed by 1)
   const T* dz = reinterpret_cast<const T*>(a.dz);
   const float skip = a.skip ? a.skip[h] : 0.f;
   const float inv_tau = MODE == 0 ? 1.f / a.tau : 0.f;
   const float rate = MODE == 1 ? expf(a.rate[h]) : 0.f;
   // a batch's inputs travel global -> registers (issued before the previous batch is computed) -> LDS (with the
   // transcendental part of the decay evaluated once per (token, channel)); two LDS buffers, one barrier per batch
-  float rq[EPT], rk[EPT], rz[EPT], vn[CH], rdt = 0.f;
+  float rq[EPT], rk[EPT], rz[EPT], vn[CH], rdt = 0.f, rdf = 0.f, mlast = 0.f;
   auto fetch = [&](int t0) {
     const int nt = min(CH, s1 - t0);
 #pragma unroll
@@ -85,10 +97,16 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
     }
     if (MODE == 1 && threadIdx.x < CH)
       rdt = (int)threadIdx.x < nt ? (float)dz[(long long)(t0 + threadIdx.x) * a.ldd + h] + a.dbias[h] : 0.f;
+    if (MODE == 2 && threadIdx.x < CH) {
+      const float* gz = reinterpret_cast<const float*>(a.dz) + (long long)(t0 + threadIdx.x) * a.ldd;
+      rdt = (int)threadIdx.x < nt ? gz[h] + a.dbias[h] : 0.f;
+      rdf = (int)threadIdx.x < nt ? gz[a.H + h] + a.dbias[a.H + h] : 0.f;
+    }
 #pragma unroll
-    for (int tt = 0; tt < CH; ++tt) vn[tt] = (tt < nt && pin) ? (float)v[(long long)(t0 + tt) * a.ldv] : 0.f;
+    for (int tt = 0; tt < CH; ++tt)
+      vn[tt] = (tt < nt && pin) ? (MODE == 2 && !vin ? 1.f : (float)v[(long long)(t0 + tt) * a.ldv]) : 0.f;
   };
-  auto commit = [&](float* buf) {
+  auto commit = [&](float* buf, int nt) {
     float* qS = buf;
     float* kS = buf + CH * LROW;
     float* aS = kS + CH * LROW;
@@ -106,13 +124,32 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
       aS[threadIdx.x] = expf(-rate * b);
       aS[CH + threadIdx.x] = b;
     }
+    if (MODE == 2 && threadIdx.x < 64) {      // the first wave: lane tt has token tt's pre-activations
+      const float cap = a.tau;
+      const float li = cap * tanhf(rdt / cap);
+      const float lf = -softplus_exact(-(cap * tanhf(rdf / cap)));
+      float ma = 0.f, mb = 0.f, mm = 0.f;
+#pragma unroll
+      for (int tt = 0; tt < CH; ++tt) {
+        const float it = __shfl(li, tt, 64), ft = __shfl(lf, tt, 64);
+        const float mn = fmaxf(ft + mrun, it);
+        const float at = expf(ft + mrun - mn), bt = expf(it - mn);
+        if ((int)threadIdx.x == tt) ma = at, mb = bt, mm = mn;
+        if (tt < nt) mrun = mn;
+      }
+      if (threadIdx.x < CH) {
+        aS[threadIdx.x] = ma;
+        aS[CH + threadIdx.x] = mb;
+        aS[2 * CH + threadIdx.x] = mm;
+      }
+    }
   };
   fetch(s0);
   int flip = 0;
   for (int t0 = s0; t0 < s1; t0 += CH, flip ^= 1) {
     const int nt = min(CH, s1 - t0);
     float* buf = lds + flip * BUF;
-    commit(buf);
+    commit(buf, nt);
     float vr[CH];
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) vr[tt] = vn[tt];
@@ -132,7 +169,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
         // 16-byte LDS reads (rows, slices and buffers all start at multiples of four floats)
         const float4* q4 = reinterpret_cast<const float4*>(qr);
         const float4* k4 = reinterpret_cast<const float4*>(kr);
-        if (MODE == 1) {
+        if (MODE >= 1) {
           u *= aS[CH + tt];
           const float at = aS[tt];
 #pragma unroll
@@ -169,12 +206,17 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
 #pragma unroll
       for (int tt = 0; tt < CH; ++tt)
         if (tt < nt) a.out[((long long)(t0 + tt) * a.H + h) * P + p] = po[tt] + skip * vr[tt];
+    if (MODE == 2) {
+      mlast = aS[2 * CH + nt - 1];
+      if (blockIdx.x == 0 && (int)threadIdx.x < nt) a.mout[(long long)(t0 + threadIdx.x) * a.H + h] = aS[2 * CH + threadIdx.x];
+    }
   }
   if (sv >= 0 && pin) {
-    float* st = a.state + (long long)sv * a.state_stride + (long long)h * N * P + p;
+    float* st = a.state + (long long)sv * a.state_stride + (long long)h * (N + (MODE == 2)) * P + p;
 #pragma unroll
     for (int i = 0; i < NPL; ++i)
       if (n0 + i < N) st[(long long)(n0 + i) * P] = S[i];
+    if (MODE == 2 && ns == 0) st[(long long)N * P] = mlast;
   }
 }
 
@@ -183,7 +225,7 @@ void launch_one(const DecayScanArgs& a, hipStream_t s) {
   const int cols = (64 / SLICES) * (NT / 64);
   dim3 grid((a.P + cols - 1) / cols, a.H, a.runs);
   const int lrow = SLICES * (NPL + 4);
-  const size_t lds = (size_t)2 * (2 * CH * lrow + (MODE == 0 ? CH * lrow : 2 * CH)) * sizeof(float);
+  const size_t lds = (size_t)2 * (2 * CH * lrow + (MODE == 0 ? CH * lrow : (MODE == 1 ? 2 : 3) * CH)) * sizeof(float);
   decay_scan_kernel<T, MODE, NPL, CH, SLICES><<<grid, NT, lds, s>>>(a);
 }
 
@@ -212,9 +254,11 @@ void launch_decay_scan(const DecayScanArgs& a, int f32, hipStream_t s) {
   if (a.runs <= 0 || a.T <= 0) return;
   if (f32) {
     if (a.mode == 0) launch_mode<float, 0>(a, s);
-    else launch_mode<float, 1>(a, s);
+    else if (a.mode == 1) launch_mode<float, 1>(a, s);
+    else launch_mode<float, 2>(a, s);
   } else {
     if (a.mode == 0) launch_mode<bf16, 0>(a, s);
-    else launch_mode<bf16, 1>(a, s);
+    else if (a.mode == 1) launch_mode<bf16, 1>(a, s);
+    else launch_mode<bf16, 2>(a, s);
   }
 }

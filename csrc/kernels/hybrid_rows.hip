@@ -100,25 +100,34 @@ __global__ __launch_bounds__(BT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
   const T* z = reinterpret_cast<const T*>(a.z) + (long long)row * a.ldz;
   const int nq = a.H * a.dk, nk = a.G * a.dk, nv = a.G * a.dv;
   const int rot = 2 * a.pairs;
-  const float* cs = a.rope + (long long)a.positions[row] * rot;   // [pairs][2]
+  const float* cs = a.rope ? a.rope + (long long)a.positions[row] * rot : nullptr;   // [pairs][2]
   const int slot = a.slots[row];
   T* qo = reinterpret_cast<T*>(a.q_out) + (long long)row * nq;
   T* kc = slot >= 0 ? reinterpret_cast<T*>(a.k_cache) + (long long)slot * nk : nullptr;
   T* vc = slot >= 0 ? reinterpret_cast<T*>(a.v_cache) + (long long)slot * nv : nullptr;
   for (int i = threadIdx.x; i < nq + nk; i += BT) {
     const int e = i < nq ? i % a.dk : (i - nq) % a.dk;   // entry within its head
-    float v = (float)z[i] + a.bias[i];
+    float v = (float)z[i] + (a.bias ? a.bias[i] : 0.f);
     if (e < rot) {
-      const int j = i - e + (e ^ 1);                     // the pair's other entry
-      const float u = (float)z[j] + a.bias[j];
-      const float c = cs[e & ~1], s = cs[(e & ~1) + 1];
-      v = (e & 1) ? v * c + u * s : v * c - u * s;
+      if (a.half) {                                      // entry e with entry e +- pairs, table pair e mod pairs
+        const bool lo = e < a.pairs;
+        const int j = lo ? i + a.pairs : i - a.pairs, pi = lo ? e : e - a.pairs;
+        const float u = (float)z[j] + (a.bias ? a.bias[j] : 0.f);
+        const float c = cs[2 * pi], s = cs[2 * pi + 1];
+        v = lo ? v * c - u * s : v * c + u * s;
+      } else {
+        const int j = i - e + (e ^ 1);                   // the pair's other entry
+        const float u = (float)z[j] + (a.bias ? a.bias[j] : 0.f);
+        const float c = cs[e & ~1], s = cs[(e & ~1) + 1];
+        v = (e & 1) ? v * c + u * s : v * c - u * s;
+      }
     }
     if (i < nq) qo[i] = (T)v;
     else if (kc) kc[i - nq] = (T)v;
   }
   if (vc)
-    for (int i = threadIdx.x; i < nv; i += BT) vc[i] = (T)((float)z[nq + nk + i] + a.bias[nq + nk + i]);
+    for (int i = threadIdx.x; i < nv; i += BT)
+      vc[i] = (T)((float)z[nq + nk + i] + (a.bias ? a.bias[nq + nk + i] : 0.f));
 }
 
 // grid (T, C / group); BT threads over the group's columns
@@ -223,11 +232,14 @@ __global__ __launch_bounds__(NT) void silu_mul_kernel(const T* __restrict__ g, l
 }
 
 // One workgroup per token: the four waves share the router outputs (a wave per output, lanes over the width), then the
-// first wave normalises and picks.  Dynamic LDS: En floats.
+// first wave normalises and picks.  Dynamic LDS: En floats.  groups > keep: the outputs form equal groups of
+// neighbours; the `keep` groups with the largest best entry (of score + correction) are picked first, and only their
+// entries can be chosen.
 template <typename T>
 __global__ __launch_bounds__(NT) void softmax_topk_kernel(const T* __restrict__ x, const T* __restrict__ Wr,
-                                                          const float* __restrict__ corr, int d, int En, int k,
-                                                          int* __restrict__ ids, float* __restrict__ w) {
+                                                          const float* __restrict__ corr, int d, int En, int k, int groups,
+                                                          int keep, int renorm, int* __restrict__ ids,
+                                                          float* __restrict__ w) {
   extern __shared__ float sc[];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* xr = x + (long long)t * d;
@@ -251,13 +263,35 @@ __global__ __launch_bounds__(NT) void softmax_topk_kernel(const T* __restrict__ 
   }
   __syncthreads();
   if (wave) return;
+  const bool grouped = groups > 1 && keep < groups;
+  const int per = grouped ? En / groups : En;
+  unsigned long long elig = ~0ull;   // bit g: group g's entries can be chosen (groups <= 64; the same in every lane)
+  if (grouped) {
+    float gbest = -INFINITY;         // lane g: the best entry of group g
+    if (lane < groups)
+      for (int e = lane * per; e < (lane + 1) * per; ++e) gbest = fmaxf(gbest, sc[e] + (corr ? corr[e] : 0.f));
+    elig = 0;
+    for (int j = 0; j < keep; ++j) {   // the keep best groups, one at a time (ties: the lowest index)
+      float best = (lane < groups && !((elig >> lane) & 1)) ? gbest : -INFINITY;
+      int bi = best > -INFINITY ? lane : 0x7fffffff;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+      }
+      if (bi < groups) elig |= 1ull << bi;
+    }
+  }
   unsigned long long taken = 0;   // bit i: this lane's entry lane + 64 i is chosen (En <= 4096)
+  float wsum = 0.f;
   for (int j = 0; j < k; ++j) {
     float best = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane, i = 0; e < En; e += 64, ++i) {
       if ((taken >> i) & 1) continue;
-      const float v = sc[e] + corr[e];
+      if (grouped && !((elig >> (e / per)) & 1)) continue;
+      const float v = sc[e] + (corr ? corr[e] : 0.f);
       if (v > best) { best = v; bi = e; }     // ascending e: the lowest index wins a tie within the lane
     }
 #pragma unroll
@@ -268,10 +302,15 @@ __global__ __launch_bounds__(NT) void softmax_topk_kernel(const T* __restrict__ 
     }
     if (bi >= En) bi = j;   // only with non-finite scores: keep the id a valid segment index for the kernels downstream
     if ((bi & 63) == lane) taken |= 1ull << (bi >> 6);
+    wsum += sc[bi];
     if (lane == 0) {
       ids[(long long)t * k + j] = bi;
       w[(long long)t * k + j] = sc[bi];
     }
+  }
+  if (renorm && lane == 0) {
+    const float den = wsum + 1e-20f;
+    for (int j = 0; j < k; ++j) w[(long long)t * k + j] = sc[ids[(long long)t * k + j]] / den;
   }
 }
 
@@ -660,11 +699,12 @@ void launch_silu_mul(const void* gate, long long ldg, const void* up, long long 
                                                                               (T*)out, R, F);)
 }
 
-void launch_softmax_topk(const void* x, const void* Wr, const float* corr, int T_, int d, int En, int k, int* ids,
-                         float* w, int f32, hipStream_t s) {
+void launch_softmax_topk(const void* x, const void* Wr, const float* corr, int T_, int d, int En, int k, int groups,
+                         int keep, int renorm, int* ids, float* w, int f32, hipStream_t s) {
   if (T_ <= 0) return;
-  DISPATCH_T(f32, softmax_topk_kernel<T><<<T_, NT, En * sizeof(float), s>>>((const T*)x, (const T*)Wr, corr, d, En, k,
-                                                                            ids, w);)
+  const size_t lds = (size_t)En * sizeof(float);
+  DISPATCH_T(f32, softmax_topk_kernel<T><<<T_, NT, lds, s>>>((const T*)x, (const T*)Wr, corr, d, En, k, groups, keep,
+                                                             renorm, ids, w);)
 }
 
 void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* w, int k, int E, const void* h,

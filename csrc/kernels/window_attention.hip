@@ -2,7 +2,9 @@
 // sigmoid output gate and an optional per-head logarithmic distance bias (the score of a key n positions back is
 // lowered by b1_h ln(1 + b2_h n)).
 //
-// Row r (position p of sequence row_seq[r]) sees positions max(0, p - window + 1) .. p; query head h reads key / value
+// Row r (position p of sequence row_seq[r]) sees positions max(0, p - window + 1) .. p and, with keep_first, the
+// sequence's first keep_first positions (at their true places in the cache); with a sink the softmax's denominator of
+// head h also holds exp(sink[h]), a logit without key or value; query head h reads key / value
 // head h / (H / G).  Key and value head sizes are independent (dk, dv).  Scores, softmax statistics, weights and the
 // weighted sum are fp32.
 //
@@ -93,6 +95,8 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
   const int nvc = vcols<PAIR>(a.dv), pstride = 2 + 64 * nvc;
   const int p = a.positions[row];
   const int j0 = max(0, p - a.window + 1);
+  // the keys of the row in walking order: the kept first positions that lie before the window, then the window
+  const int kf = min(a.keep_first, j0), total = kf + p - j0 + 1;
   const int* bt = a.block_tables + (long long)a.row_seq[row] * a.max_blocks;
   const T* q = reinterpret_cast<const T*>(a.q) + ((long long)row * a.H + h0) * a.dk;   // REP heads: contiguous
   for (int e = threadIdx.x; e < REP * a.dk; e += 64 * NW) qs[e] = (float)q[e] * a.scale;
@@ -109,11 +113,13 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
 #pragma unroll
     for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] = 0.f;
   }
-  for (int t0 = j0 + 64 * wave; t0 <= p; t0 += 64 * NW) {
-    const int j = t0 + lane;
+  for (int t0 = 64 * wave; t0 < total; t0 += 64 * NW) {
+    const int idx = t0 + lane;
+    const bool on = idx < total;
+    const int j = idx < kf ? idx : j0 + idx - kf;
     float sc[REP], w[REP];
-    long long slot = 0;                       // lanes past the row's position: weight 0 on a finite row (slot 0)
-    if (j <= p) {
+    long long slot = 0;                       // lanes past the row's last key: weight 0 on a finite row (slot 0)
+    if (on) {
       slot = cache_row(bt, j, a.BS, a.bs_shift);
       dot_rows<T, REP>(kc + (slot * a.G + g) * a.dk, qs, a.dk, sc);
       if (a.bias) {
@@ -126,16 +132,16 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     }
 #pragma unroll
     for (int r = 0; r < REP; ++r) {
-      const float s = j <= p ? sc[r] : -INFINITY;
+      const float s = on ? sc[r] : -INFINITY;
       const float mt = fmaxf(m[r], wave_max(s));
-      w[r] = j <= p ? expf(s - mt) : 0.f;
+      w[r] = on ? expf(s - mt) : 0.f;
       const float corr = expf(m[r] - mt);     // first tile: exp(-inf) = 0 on an all-zero accumulator
       l[r] = l[r] * corr + wave_sum(w[r]);
       m[r] = mt;
 #pragma unroll
       for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] *= corr;
     }
-    const int nt = min(64, p - t0 + 1);
+    const int nt = min(64, total - t0);
     const int vslot = (int)slot;              // (cache rows fit 31 bits: checked by the op layer)
     // value rows VB at a time: their cache rows come lane by lane from the scoring phase (no block-table walk in this
     // loop), the loads of a batch are issued together and serve all REP heads
@@ -199,6 +205,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
       float M = m[r];
       for (int w2 = 1; w2 < NW; ++w2) M = fmaxf(M, part[(w2 * REP + r) * pstride]);
       const float f0 = expf(m[r] - M);
+      m[r] = M;
       l[r] *= f0;
 #pragma unroll
       for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] *= f0;
@@ -219,6 +226,12 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     if (a.gate) {
       const float gv = (float)reinterpret_cast<const T*>(a.gate)[(long long)row * a.ldg + h];
       gate = 1.f / (1.f + expf(-gv));
+    }
+    if (a.sink) {     // one more term in the denominator: exp(sink - M) with M = max(m, sink)
+      const float sk = a.sink[h], M = fmaxf(m[r], sk);
+      const float f = expf(m[r] - M);
+      l[r] = l[r] * f + expf(sk - M);
+      gate *= f;
     }
     const float inv = gate / l[r];
     T* o = reinterpret_cast<T*>(a.out) + ((long long)row * a.H + h) * a.dv;
@@ -306,10 +319,15 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
   // cache blocks of 64 tokens or a multiple: a key tile lies in one block, whose number is read one tile ahead (the
   // rows' loads then do not wait for a block-table load of their own)
   const bool one_block = a.bs_shift >= 6;
-  int blk_next = one_block ? bt[(k_lo & ~63) >> a.bs_shift] : 0;
-  for (int kt = k_lo & ~63; kt <= p_last; kt += 64) {
+  // key tiles in walking order: the tiles of the kept first positions that lie before the window's first tile, then the
+  // window's tiles up to the last row's own position
+  const int kt_win = k_lo & ~63;
+  const int kt_first = (a.keep_first > 0 && kt_win > 0) ? 0 : kt_win;
+  auto tile_after = [&](int kt) { return (kt < kt_win && kt + 64 >= min(a.keep_first, kt_win)) ? kt_win : kt + 64; };
+  int blk_next = one_block ? bt[kt_first >> a.bs_shift] : 0;
+  for (int kt = kt_first; kt <= p_last; kt = tile_after(kt)) {
     const long long blk_base = (long long)blk_next << (one_block ? a.bs_shift : 0);
-    if (one_block && kt + 64 <= p_last) blk_next = bt[(kt + 64) >> a.bs_shift];
+    if (one_block && tile_after(kt) <= p_last) blk_next = bt[tile_after(kt) >> a.bs_shift];
     auto row_of = [&](int kp) {
       return one_block ? blk_base + (kp & (a.BS - 1)) : cache_row(bt, kp, a.BS, a.bs_shift);
     };
@@ -352,7 +370,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
     // scores in units of log2(e): sc[s][e] = scale * log2(e) * q_j . k_(kt + 16 s + 4 hq + e).  A key tile that every
     // row of the wave sees completely (the usual case away from the diagonal and the window's far edge) skips the masks.
     const int wq_lo = p_first + 16 * wave, wq_hi = wq_lo + 15;
-    const bool interior = 16 * wave + 15 < nrows && kt + 63 <= wq_lo && kt > wq_hi - a.window;
+    const bool interior = 16 * wave + 15 < nrows && kt + 63 <= wq_lo && (kt > wq_hi - a.window || kt + 63 < a.keep_first);
     float pv[4][4];
     float mx = -INFINITY;
     // 1 + b2 (qp - kp) for key kp = kt + 16 s4 + 4 hq + e is arg0 - b2 (16 s4 + e): one multiply-add per score
@@ -377,7 +395,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int kp = kt + 16 * s4 + 4 * hq + e;
-          const bool vis = rv && kp <= qp && kp > qp - a.window;
+          const bool vis = rv && kp <= qp && (kp > qp - a.window || kp < a.keep_first);
           float sv = acc[e] * sl2;
           if (biased) sv += nb1 * __log2f(arg0 - b2 * (float)(16 * s4 + e));   // (keys past the row: masked below)
           pv[s4][e] = vis ? sv : -INFINITY;
@@ -431,6 +449,12 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
   if (a.gate) {
     const float gv = (float)reinterpret_cast<const bf16*>(a.gate)[(long long)my_row * a.ldg + h];
     gate = 1.f / (1.f + expf(-gv));
+  }
+  if (a.sink) {     // one more term in the denominator (m is in units of log2 e)
+    const float sk = a.sink[h] * 1.44269504088896341f, M = fmaxf(m, sk);
+    const float f = exp2f(m - M);
+    l = l * f + exp2f(sk - M);
+    gate *= f;
   }
   const float inv = gate / l;
   bf16* out = reinterpret_cast<bf16*>(a.out) + ((long long)my_row * a.H + h) * DV + 4 * hq;

@@ -50,7 +50,7 @@ LATENT_BINDINGS = ("latent_ops.cpp",)
 # feed-forward with a softmax router) and their op bindings; the routed feed-forward shares glu_moe.hip's expert-segment
 # kernels, so that translation unit is linked into both libraries
 HYBRID_SO = os.path.join(PKG, "_C_hybrid.so")
-HYBRID_KERNELS = ("hybrid_rows.hip", "window_attention.hip", "decay_scan.hip")
+HYBRID_KERNELS = ("hybrid_rows.hip", "stream_rows.hip", "window_attention.hip", "decay_scan.hip")
 HYBRID_SHARED = ("glu_moe.hip",)
 HYBRID_BINDINGS = ("hybrid_ops.cpp",)
 NET_SO = os.path.join(PKG, "net", "_native.so")
@@ -184,7 +184,7 @@ def build_latent(verbose: bool = False, force: bool = False) -> str:
 
 
 def build_hybrid(verbose: bool = False, force: bool = False) -> str:
-    """csrc/kernels/{hybrid_rows,window_attention,decay_scan,glu_moe}.hip + csrc/bindings/hybrid_ops.cpp ->
+    """csrc/kernels/{hybrid_rows,stream_rows,window_attention,decay_scan,glu_moe}.hip + csrc/bindings/hybrid_ops.cpp ->
     symmetry_amd/_C_hybrid.so (``torch.ops.symmetry_amd_hybrid``)."""
     os.makedirs(OBJ, exist_ok=True)
     kdir = os.path.join(CSRC, "kernels")

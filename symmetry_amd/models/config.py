@@ -845,7 +845,7 @@ class DalalixConfig:
         for layer in self.layers:
             m = layer.mixer
             if layer.type == "parallel":
-                n += m.right.heads * (m.right.dim * (m.right.vdim + 1) + 1) * 4
+                n += m.right.heads * (m.right.dim + 1) * (m.right.vdim + 1) * 4
             elif m.conv > 1:
                 n += (m.conv - 1) * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) * dtype_bytes
         return n

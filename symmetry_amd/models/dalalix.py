@@ -60,13 +60,13 @@ class DalalixCache:
     ``k`` / ``v``: one pair of paged planes per layer, [NB, BS, G, dk] / [NB, BS, G, dv] (token-major), on the engine's
     BlockManager numbering (one block table serves all planes).  Per state slot: ``tok`` the sequence's last token
     (int32), ``conv`` per convolving layer the newest taps - 1 projected rows [slots, taps - 1, C], ``mem`` per matrix
-    memory [slots, H, N, P + 1] fp32 (the last column is the normaliser) and ``mmax`` its running maximum [slots, H].
+    memory [slots, H, N + 1, P + 1] fp32 (the last column is the normaliser, the last row the running maximum).
     Slots are handed out by the scheduler's StateSlotManager; a slot's old content is never read by a new sequence (its
     first run starts from zero).  Zero-initialised: every byte finite."""
 
     def __init__(self, cfg: DalalixConfig, num_blocks: int, block_size: int, num_slots: int, device, dtype):
         self.num_layers, self.num_blocks, self.block_size = cfg.num_layers, num_blocks, block_size
-        self.k, self.v, self.conv, self.mem, self.mmax = {}, {}, {}, {}, {}
+        self.k, self.v, self.conv, self.mem = {}, {}, {}, {}
         self.tok = torch.zeros(num_slots, device=device, dtype=torch.int32)
         for i, layer in enumerate(cfg.layers):
             a = cfg.attn_spec(i)
@@ -74,15 +74,14 @@ class DalalixCache:
             self.v[i] = torch.zeros(num_blocks, block_size, a.kv_heads, a.vdim, device=device, dtype=dtype)
             if layer.type == "parallel":
                 g = layer.mixer.right
-                self.mem[i] = torch.zeros(num_slots, g.heads, g.dim, g.vdim + 1, device=device, dtype=torch.float32)
-                self.mmax[i] = torch.zeros(num_slots, g.heads, device=device, dtype=torch.float32)
+                self.mem[i] = torch.zeros(num_slots, g.heads, g.dim + 1, g.vdim + 1, device=device, dtype=torch.float32)
             elif a.conv:
                 C = a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)
                 self.conv[i] = torch.zeros(num_slots, a.conv - 1, C, device=device, dtype=dtype)
 
     def nbytes(self) -> int:
         return self.tok.numel() * 4 + sum(t.numel() * t.element_size()
-                                          for d in (self.k, self.v, self.conv, self.mem, self.mmax) for t in d.values())
+                                          for d in (self.k, self.v, self.conv, self.mem) for t in d.values())
 
 
 class DalalixLM:
@@ -296,7 +295,7 @@ class DalalixLM:
         ops.decay_scan(ops.DECAY_LOG_GATES, self._cols(z, P, "right.q"), self._cols(z, P, "right.k"),
                        self._cols(z, P, "right.v"), gates, P["right.gates.b"], g.gate_cap, None, g.dim ** -0.5, g.heads,
                        g.dim, g.vdim, 1, cache.mem[i], b.cu_q if prefill else None, b.prev_row, b.save_slot, runs, y,
-                       mstate=cache.mmax[i], mout=mx)
+                       mout=mx)
         gy = self._buf("mem.gy", (T, g.heads * g.vdim))
         ops.memory_norm_gate(y, mx, self._cols(z, P, "right.g"), P["right.norm"], self.cfg.norm_eps, gy)
         right = self._linear("mem.out", gy, P["right.o"])

@@ -786,24 +786,25 @@ DECAY_CHANNEL_GATE, DECAY_STEP_SIZE, DECAY_LOG_GATES = 0, 1, 2
 
 
 def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
-               out, mstate=None, mout=None):
+               out, mout=None):
     """Linear recurrence with decaying state, per head h over every run of rows (cu_q[i] .. cu_q[i + 1]; cu_q None:
     every row its own run): S <- diag(a_t) S + b_t k_t v_t^T (S [N, P] fp32), out_t = S^T (q_scale q_t) (+ skip_h v_t).
     DECAY_CHANNEL_GATE: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel (dz [T, H N], dparam a number), b = 1;
     DECAY_STEP_SIZE: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) b) per head (dz [T, H]).
     DECAY_LOG_GATES: dz fp32 [T, 2 H] = input | forget pre-activations, dbias [2 H], dparam the gates' soft cap c:
     i = c tanh(. / c), f = logsigmoid(c tanh(. / c)), running maximum m_t = max(f + m_(t-1), i) (0 at a sequence's start,
-    carried in mstate [slots, H], written to mout [T, H]), a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); state
-    [slots, H, N, P + 1] and out [T, H, P + 1] carry one more column, fed by v = 1 (the normaliser n_t and n_t . q_t).
+    written to mout [T, H]), a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); state [slots, H, N + 1, P + 1] and out
+    [T, H, P + 1] carry one more column, fed by v = 1 (the normaliser n_t and n_t . q_t), and the state one more row,
+    which carries m (the same value in every column).
     q / k [T, (H / hpg) N]: head h reads group h // hpg.  A run starts from state[slot] if prev_row[first] <= -2
     (slot = -(v + 2)), else from zero; it ends in state[save_slot[last]] (>= 0).  out fp32 [T, H, P]."""
     if _gpu(out):
         dp = dparam if torch.is_tensor(dparam) else None
         return _hyb().decay_scan(int(mode), q, k, v, dz, dbias, dp, 0.0 if dp is not None else float(dparam), skip,
                                  float(q_scale), int(H), int(N), int(P), int(hpg), state, cu_q, prev_row, save_slot,
-                                 int(runs), out, mstate, mout)
+                                 int(runs), out, mout)
     return reference.decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row,
-                                save_slot, runs, out, mstate, mout)
+                                save_slot, runs, out, mout)
 
 
 def memory_norm_gate(y, m, gate, w, eps, out):

@@ -827,13 +827,14 @@ def _runs(T, cu_q, runs):
 
 
 def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
-               out, mstate=None, mout=None) -> None:
+               out, mout=None) -> None:
     """S <- diag(a_t) S + b_t k_t v_t^T, o_t = S^T (q_scale q_t) (+ skip_h v_t) per head over every run of rows.
     mode 0: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel, b = 1;
     mode 1: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) * b) per head.  q / k of head h: group h // hpg.
     mode 2: log gates i = c tanh((dz[:, h] + dbias[h]) / c), f = logsigmoid(c tanh((dz[:, H + h] + dbias[H + h]) / c)),
-    c = dparam; running maximum m_t = max(f + m_(t-1), i) (carried in mstate, 0 at a sequence's start, written to mout);
-    a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); the state and the output have one more column, fed by v = 1."""
+    c = dparam; running maximum m_t = max(f + m_(t-1), i) (0 at a sequence's start, written to mout); a = exp(f + m_(t-1)
+    - m_t), b = exp(i - m_t); the state and the output have one more column, fed by v = 1, and the state one more row
+    that carries m (the same value in every column)."""
     T = q.shape[0]
     qf = q.float().reshape(T, -1, N) * q_scale
     kf, vf = k.float().reshape(T, -1, N), v.float().reshape(T, H, P)
@@ -856,9 +857,9 @@ def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, st
         if s1 <= s0:
             continue
         pr = int(prev_row[s0])
-        S = state[-(pr + 2)].clone() if pr <= -2 else torch.zeros(H, N, P)
+        S = state[-(pr + 2)][:, :N].clone() if pr <= -2 else torch.zeros(H, N, P)
         if mode == 2:
-            m = mstate[-(pr + 2)].clone() if pr <= -2 else torch.zeros(H)
+            m = state[-(pr + 2)][:, N, 0].clone() if pr <= -2 else torch.zeros(H)
         for t in range(s0, s1):
             if mode == 2:
                 mn = torch.maximum(lf[t] + m, li[t])
@@ -874,9 +875,9 @@ def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, st
             o[t] = y
         sv = int(save_slot[s1 - 1])
         if sv >= 0:
-            state[sv] = S
+            state[sv][:, :N] = S
             if mode == 2:
-                mstate[sv] = m
+                state[sv][:, N] = m[:, None]
 
 
 def memory_norm_gate(y, m, gate, w, eps, out) -> None:
