@@ -161,7 +161,9 @@ def matrix_memory(W, p, m, h, eps):
 def route(z, top, groups, keep):
     """Router: softmax over all experts; experts form ``groups`` equal groups of neighbours, a group scores as its best
     expert, only the ``keep`` best groups stay eligible; the ``top`` best eligible experts, weights = their scores over
-    their sum.  z [E] -> (ids, weights, margin between the last chosen and the best one left out)."""
+    their sum.  z [E] -> (ids, weights, margin).  The margin says how far the choice is from another one, in units of the
+    logits: the last chosen expert against the best eligible one left out, and the last kept group against the best one
+    dropped; infinite where the expert that a flip would swap carries next to no weight."""
     s = torch.softmax(z, -1)
     E = s.shape[0]
     per = E // groups
@@ -172,14 +174,18 @@ def route(z, top, groups, keep):
         ok[g * per:(g + 1) * per] = True
     masked = torch.where(ok, s, torch.full_like(s, -1.0))
     val, ids = torch.topk(masked, top)
-    rest = masked.clone()
-    rest[ids] = -1.0
-    margin = float(val[-1] - rest.max()) if top < E else 1.0
-    if keep < groups:
-        gl = gs.clone()
-        gl[kept] = -1.0
-        margin = min(margin, float(gs[kept].min() - gl.max()))
     w = s[ids] / (s[ids].sum() + 1e-20)
+    margin = math.inf
+    if float(w[-1]) > 0.03:
+        rest = torch.where(ok, z, torch.full_like(z, -math.inf))
+        rest[ids] = -math.inf
+        if top < int(ok.sum()):
+            margin = float(z[ids[-1]] - rest.max())
+        if keep < groups:
+            gz = z.view(groups, per).max(-1).values
+            gl = gz.clone()
+            gl[kept] = -math.inf
+            margin = min(margin, float(gz[kept].min() - gl.max()))
     return ids, w, margin
 
 
@@ -194,12 +200,14 @@ def moe(W, p, f, h, margins=None):
     grp = r.get("groups") or {"count": 1, "keep": 1}
     z = h @ W[p + "router"].T
     out = torch.zeros_like(h)
+    ms = []
     for t in range(h.shape[0]):
         ids, w, mg = route(z[t], r["top"], grp["count"], grp["keep"])
-        if margins is not None:
-            margins.append(mg)
+        ms.append(mg)
         for e, we in zip(ids.tolist(), w):
             out[t] += we * expert(W, f"{p}e{e}.", h[t], f["expert"]["limit"])
+    if margins is not None:
+        margins.append(torch.tensor(ms))
     return out
 
 
@@ -219,7 +227,7 @@ def mixer(W, cfg, L, p, h, positions):
 
 def forward(W, cfg, tokens, layers_out=None, margins=None):
     """Logits [T, vocab] of one sequence, float64.  ``layers_out`` (a list) receives the sum of the streams after every
-    layer; ``margins`` the routers' margins (see ``route``)."""
+    layer; ``margins`` one tensor [T] per routed sublayer: the routers' margins (see ``route``)."""
     W = {k: v.to(F64) for k, v in W.items()}
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     T = tokens.shape[0]
