@@ -604,7 +604,7 @@ def test_windowed_attention_keeps_first_tokens_and_a_sink(device, dtype):
             assert float((wide - want[149:]).abs().max()) > 50 * tol, target
     nosink = torch.empty(1, H, dv, dtype=dtype, device=device)
     ops.window_attn(qd[100:101], kcd, vcd, btd, rsd[:1], posd[100:101], window, 0.3, None, nosink, keep_first=keep)
-    assert float((nosink.cpu().double() - want[100:101]).abs().max()) > 50 * tol      # (a row that looks at no key hard)
+    assert float((nosink.cpu().double() - want[100:101]).abs().max()) > 0.02      # (a row that looks at no key hard)
 
 
 @pytest.mark.parametrize("device", DEVICES)
