@@ -72,10 +72,10 @@ def _args():
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--families", action="store_true",
                     help="instead of the serving benchmark: prefill / decode throughput of Bozevik (or, with "
-                         "--family-design lemunex / komazen, Lemunex / Komazen) stacks beside the closest Llama / Mixtral "
+                         "--family-design lemunex / komazen / dalalix, those) stacks beside the closest Llama / Mixtral "
                          "stacks of equal size (bench/families.py; one GPU)")
     ap.add_argument("--family-sizes", default="w2048,w4096,moe-w2048")
-    ap.add_argument("--family-design", default="bozevik", choices=("bozevik", "lemunex", "komazen"))
+    ap.add_argument("--family-design", default="bozevik", choices=("bozevik", "lemunex", "komazen", "dalalix"))
     ap.add_argument("--nt-weights", type=int, default=None, help="A/B: non-temporal decode weight loads (0/1)")
     ap.add_argument("--max-batched-tokens", type=int, default=None, help="A/B: token budget of a pure-prefill step")
     ap.add_argument("--mixed-prefill-tokens", type=int, default=None, help="A/B: prompt budget of mixed steps")

@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a Bozevik, Lemunex or Komazen stack beside the closest Llama / Mixtral stack of equal
-size.
+"""Prefill and decode throughput of a Bozevik, Lemunex, Komazen or Dalalix stack beside the closest Llama / Mixtral stack
+of equal size.
 
 Random weights, layer shapes of real models, a few layers each (throughput per layer is what is compared; the
 vocabulary projection is the same size on both sides).  Per size and family, through the engine's own scheduler:
@@ -84,6 +84,32 @@ def _komazen_pairs():
     }
 
 
+def _dalalix_pairs():
+    """Dalalix stacks (causal attention with biased projections, windowed attention with kept first tokens and a sink
+    beside a matrix memory, two causal layers with convolved projections; four residual streams; routed clamped experts
+    with group-limited choice) beside the Mixtral stack of the same width, head count, expert count and expert width, and
+    beside the Lemunex stack with routed layers (the closest model with a recurrence beside windowed attention); the
+    window equals the benchmark's prompt length."""
+    from symmetry_amd.models.config import ModelConfig, dalalix_stack, lemunex_stack
+
+    kw = dict(max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+    dk = dict(window=1024, keep_first=4, groups=4, keep=2, streams=4, buckets=65521, conv=4)
+    return {
+        "w2048": (dalalix_stack("dalalix-w2048", 32768, 2048, "BPCC", heads=16, kv_heads=4, dim=128, experts=16, top=4,
+                                expert_ff=1536, mem_heads=8, mem_dim=128, mem_vdim=256, **dk, **kw),
+                  ModelConfig("mixtral-w2048", 32768, 2048, 1536, 4, 16, 4, num_experts=16, top_k=4, **kw)),
+        "w4096": (dalalix_stack("dalalix-w4096", 32768, 4096, "BPCC", heads=32, kv_heads=8, dim=128, experts=8, top=2,
+                                expert_ff=14336, mem_heads=16, mem_dim=128, mem_vdim=256, **{**dk, "groups": 2, "keep": 1},
+                                **kw),
+                  ModelConfig("mixtral-w4096", 32768, 4096, 14336, 4, 32, 8, num_experts=8, top_k=2, **kw)),
+        "moe-w2048": (dalalix_stack("dalalix-w2048", 32768, 2048, "BPCC", heads=16, kv_heads=4, dim=128, experts=16, top=4,
+                                    expert_ff=1536, mem_heads=8, mem_dim=128, mem_vdim=256, **dk, **kw),
+                      lemunex_stack("lemunex-moe", 32768, 2048, "PMMP", heads=16, kv_heads=4, dim=128, window=1024,
+                                    gla_heads=8, gla_dim=128, gla_vdim=256, ssm_heads=64, ssm_vdim=64, ssm_state=128,
+                                    ff=8192, experts=16, top=4, identity=2, expert_ff=1024, shared_ff=2048, **kw)),
+    }
+
+
 def measure(mcfg, prompts: int, plen: int, steps: int, reps: int = 3) -> dict:
     import torch
 
@@ -135,10 +161,11 @@ def main(argv=None) -> int:
     ap.add_argument("--prompts", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--decode-steps", type=int, default=64)
-    ap.add_argument("--only", default="", help="bozevik | lemunex | komazen | baseline: one side only (profiling)")
-    ap.add_argument("--design", default="bozevik", choices=("bozevik", "lemunex", "komazen"), help="the family measured")
+    ap.add_argument("--only", default="", help="bozevik | lemunex | komazen | dalalix | baseline: one side only (profiling)")
+    ap.add_argument("--design", default="bozevik", choices=("bozevik", "lemunex", "komazen", "dalalix"),
+                    help="the family measured")
     a = ap.parse_args(argv)
-    pairs = {"bozevik": _pairs, "lemunex": _lemunex_pairs, "komazen": _komazen_pairs}[a.design]()
+    pairs = {"bozevik": _pairs, "lemunex": _lemunex_pairs, "komazen": _komazen_pairs, "dalalix": _dalalix_pairs}[a.design]()
     ratios = {}
     for size in a.sizes.split(","):
         if size not in pairs:     # (a design without routed layers has no routed size)

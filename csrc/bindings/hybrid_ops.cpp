@@ -716,11 +716,11 @@ void conv_qkv_cache(const Tensor& z, const Tensor& w, Tensor& state, const OptTe
   dtype(prev_row, at::kInt, "prev_row");
   dtype(slots, at::kInt, "slots");
   const int64_t taps = w.size(1);
-  TORCH_CHECK(w.size(0) == C && taps >= 1 && taps <= 16 && state.size(1) == taps - 1 && state.size(2) == C && C <= 15000 &&
-                  H % G == 0 && q_out.numel() == T * H * dk && prev_row.numel() >= T && slots.numel() >= T &&
-                  k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(2) == G && k_cache.size(3) == dk &&
-                  v_cache.size(2) == G && v_cache.size(3) == dv && T <= 65535 * 1024,
-              "conv_qkv_cache: shapes (at most 16 taps, 15000 channels)");
+  TORCH_CHECK(w.size(0) == C && taps >= 1 && taps <= 16 && state.size(1) == taps - 1 && state.size(2) == C && dk <= 512 &&
+                  dv <= 512 && H + 2 * G <= 65535 && H % G == 0 && q_out.numel() == T * H * dk && prev_row.numel() >= T &&
+                  slots.numel() >= T && k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(2) == G &&
+                  k_cache.size(3) == dk && v_cache.size(2) == G && v_cache.size(3) == dv && T <= 65535 * 1024,
+              "conv_qkv_cache: shapes (at most 16 taps, heads at most 512 wide)");
   if (cu_q.has_value()) {
     TORCH_CHECK(row_seq.has_value(), "conv_qkv_cache: cu_q without row_seq");
     dtype(*cu_q, at::kInt, "cu_q");

@@ -128,18 +128,19 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
       const float cap = a.tau;
       const float li = cap * tanhf(rdt / cap);
       const float lf = -softplus_exact(-(cap * tanhf(rdf / cap)));
-      float ma = 0.f, mb = 0.f, mm = 0.f;
+      // the chain m_t = max(f_t + m_(t-1), i_t) is an add and a max per token; lane tt keeps its token's pair
+      // (m_(t-1), m_t) and evaluates the two exponentials afterwards, all lanes at once
+      float mp = 0.f, mm = 0.f;
 #pragma unroll
       for (int tt = 0; tt < CH; ++tt) {
         const float it = __shfl(li, tt, 64), ft = __shfl(lf, tt, 64);
         const float mn = fmaxf(ft + mrun, it);
-        const float at = expf(ft + mrun - mn), bt = expf(it - mn);
-        if ((int)threadIdx.x == tt) ma = at, mb = bt, mm = mn;
+        if ((int)threadIdx.x == tt) mp = mrun, mm = mn;
         if (tt < nt) mrun = mn;
       }
       if (threadIdx.x < CH) {
-        aS[threadIdx.x] = ma;
-        aS[CH + threadIdx.x] = mb;
+        aS[threadIdx.x] = expf(lf + mp - mm);
+        aS[CH + threadIdx.x] = expf(li - mm);
         aS[2 * CH + threadIdx.x] = mm;
       }
     }

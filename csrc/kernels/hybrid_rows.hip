@@ -231,6 +231,38 @@ __global__ __launch_bounds__(NT) void silu_mul_kernel(const T* __restrict__ g, l
   }
 }
 
+// x . w over d entries by one wave: 16-byte loads, several in flight (a decode step has a handful of rows, so the
+// latency of a load after a load is what such a launch costs); any width and alignment through the scalar tail
+template <typename T>
+SYM_DEV float wave_dot(const T* __restrict__ x, const T* __restrict__ w, int d, int lane) {
+  float acc = 0.f;
+  int done = 0;
+  if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) == 0) {
+    if constexpr (sizeof(T) == 2) {
+      const int nv = d >> 3;
+#pragma unroll 4
+      for (int i = lane; i < nv; i += 64) {
+        float a[8], b[8];
+        load8(reinterpret_cast<const bf16*>(x) + 8 * i, a);
+        load8(reinterpret_cast<const bf16*>(w) + 8 * i, b);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += a[j] * b[j];
+      }
+      done = nv << 3;
+    } else {
+      const int nv = d >> 2;
+#pragma unroll 4
+      for (int i = lane; i < nv; i += 64) {
+        const float4 a = reinterpret_cast<const float4*>(x)[i], b = reinterpret_cast<const float4*>(w)[i];
+        acc += a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w;
+      }
+      done = nv << 2;
+    }
+  }
+  for (int c = done + lane; c < d; c += 64) acc += (float)x[c] * (float)w[c];
+  return wave_sum(acc);
+}
+
 // One workgroup per token: the four waves share the router outputs (a wave per output, lanes over the width), then the
 // first wave normalises and picks.  Dynamic LDS: En floats.  groups > keep: the outputs form equal groups of
 // neighbours; the `keep` groups with the largest best entry (of score + correction) are picked first, and only their
@@ -244,10 +276,7 @@ __global__ __launch_bounds__(NT) void softmax_topk_kernel(const T* __restrict__ 
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* xr = x + (long long)t * d;
   for (int e = wave; e < En; e += NT / 64) {
-    const T* wr = Wr + (long long)e * d;
-    float acc = 0.f;
-    for (int c = lane; c < d; c += 64) acc += (float)xr[c] * (float)wr[c];
-    acc = wave_sum(acc);
+    const float acc = wave_dot<T>(xr, Wr + (long long)e * d, d, lane);
     if (lane == 0) sc[e] = acc;
   }
   __syncthreads();

@@ -6,6 +6,7 @@
 //   hyper_mix_norm       streams <- streams M + c_out y (all at once), and the next sublayer's input rms_norm(c_in . streams)
 //                        from the same pass; also the plain gathered sum + norm in front of the output head
 //   conv_qkv_cache       causal per-channel convolution of q | k | v with carried taps, unit-RMS value heads, paged cache write
+//                        (a workgroup per (row, head))
 //   memory_norm_gate     o / (max(|n . q|, exp(-m)) + 1e-6), unit RMS per head, weight, sigmoid gate
 //   logit_softcap        cap tanh(logits / cap)
 //
@@ -138,11 +139,34 @@ __global__ __launch_bounds__(BT) void hyper_mix_norm_kernel(HyperMixArgs a) {
   for (int c = threadIdx.x; c < d; c += BT) out[c] = (T)(us[c] * r * a.w[c]);
 }
 
-// One workgroup per row, dynamic LDS C floats: the convolved row, then q / k copied out and the value heads normalised.
+// grid (T, H + 2 G): one workgroup of CQ threads per (row, head of q | k | v), a thread per channel (wider heads: several).
+// A value head is brought to unit RMS before it is stored.  The small workgroups give a decode step's few rows a few
+// hundred of them; a thread's taps and carried inputs are loads that do not depend on one another.
+constexpr int CQ = 128;
+constexpr int CQ_PER = 4;     // channels per thread kept in registers: heads up to 512 wide
 template <typename T>
-__global__ __launch_bounds__(NT) void conv_qkv_cache_kernel(ConvQkvArgs a) {
-  extern __shared__ float ys[];
-  const int row = blockIdx.x, C = a.C, taps = a.taps;
+__global__ __launch_bounds__(CQ) void conv_qkv_cache_kernel(ConvQkvArgs a) {
+  __shared__ float scratch[CQ / 64];
+  const int row = blockIdx.x, unit = blockIdx.y, C = a.C, taps = a.taps;
+  const int nq = a.H * a.dk, nk = a.G * a.dk;
+  // the unit's channels [c0, c0 + width) and where they go
+  int c0, width;
+  T* dst_out;
+  const int slot = a.slots[row];
+  bool vhead = false;
+  if (unit < a.H) {
+    c0 = unit * a.dk, width = a.dk;
+    dst_out = reinterpret_cast<T*>(a.q_out) + (long long)row * nq + c0;
+  } else if (unit < a.H + a.G) {
+    const int g = unit - a.H;
+    c0 = nq + g * a.dk, width = a.dk;
+    dst_out = slot >= 0 ? reinterpret_cast<T*>(a.k_cache) + (long long)slot * nk + g * a.dk : nullptr;
+  } else {
+    const int g = unit - a.H - a.G;
+    c0 = nq + nk + g * a.dv, width = a.dv;
+    dst_out = slot >= 0 ? reinterpret_cast<T*>(a.v_cache) + ((long long)slot * a.G + g) * a.dv : nullptr;
+    vhead = true;
+  }
   const int s0 = a.cu_q ? a.cu_q[a.row_seq[row]] : row;
   const int j = row - s0;
   const int pr = a.prev_row[s0];
@@ -151,44 +175,44 @@ __global__ __launch_bounds__(NT) void conv_qkv_cache_kernel(ConvQkvArgs a) {
   const T* w = reinterpret_cast<const T*>(a.w);
   const int sv = (!a.cu_q && a.save_slot) ? a.save_slot[row] : -1;
   T* dst = sv >= 0 ? reinterpret_cast<T*>(a.state) + (long long)sv * a.state_stride : nullptr;
-  for (int c = threadIdx.x; c < C; c += NT) {
-    float acc = 0.f;
-    for (int i = 0; i < taps; ++i) {       // i positions back
-      float v = 0.f;
-      if (i <= j) v = (float)z[(long long)(row - i) * a.ldz + c];
-      else if (st) v = (float)st[(long long)(taps - 1 - (i - j)) * C + c];
-      acc += (float)w[(long long)c * taps + taps - 1 - i] * v;
-    }
-    ys[c] = acc;
-    // rows that are runs of their own: this thread alone reads and writes its channel of the row's slot, so the carried
-    // taps move on here (older ones one place down, the row's input on top)
-    if (dst && taps > 1) {
-      const int keep = taps - 1;
-      T vals[MAX_TAPS];
+  float y[CQ_PER];
+  float sq = 0.f;
 #pragma unroll
-      for (int m = 0; m < MAX_TAPS; ++m)
-        if (m < keep) vals[m] = m + 1 < keep ? (st ? st[(long long)(m + 1) * C + c] : (T)0.f) : z[(long long)row * a.ldz + c];
+  for (int u = 0; u < CQ_PER; ++u) {
+    const int e = threadIdx.x + u * CQ;
+    y[u] = 0.f;
+    if (e < width) {
+      const int c = c0 + e;
+      float acc = 0.f;
+      for (int i = 0; i < taps; ++i) {       // i positions back
+        float v = 0.f;
+        if (i <= j) v = (float)z[(long long)(row - i) * a.ldz + c];
+        else if (st) v = (float)st[(long long)(taps - 1 - (i - j)) * C + c];
+        acc += (float)w[(long long)c * taps + taps - 1 - i] * v;
+      }
+      y[u] = acc;
+      sq += acc * acc;
+      // rows that are runs of their own: this thread alone reads and writes its channel of the row's slot, so the
+      // carried taps move on here (older ones one place down, the row's input on top)
+      if (dst && taps > 1) {
+        const int keep = taps - 1;
+        T vals[MAX_TAPS];
 #pragma unroll
-      for (int m = 0; m < MAX_TAPS; ++m)
-        if (m < keep) dst[(long long)m * C + c] = vals[m];
+        for (int m = 0; m < MAX_TAPS; ++m)
+          if (m < keep) vals[m] = m + 1 < keep ? (st ? st[(long long)(m + 1) * C + c] : (T)0.f) : z[(long long)row * a.ldz + c];
+#pragma unroll
+        for (int m = 0; m < MAX_TAPS; ++m)
+          if (m < keep) dst[(long long)m * C + c] = vals[m];
+      }
     }
   }
-  __syncthreads();
-  const int nq = a.H * a.dk, nk = a.G * a.dk, nv = a.G * a.dv;
-  const int slot = a.slots[row];
-  T* qo = reinterpret_cast<T*>(a.q_out) + (long long)row * nq;
-  for (int c = threadIdx.x; c < nq; c += NT) qo[c] = (T)ys[c];
-  if (slot < 0) return;
-  T* kc = reinterpret_cast<T*>(a.k_cache) + (long long)slot * nk;
-  T* vc = reinterpret_cast<T*>(a.v_cache) + (long long)slot * nv;
-  for (int c = threadIdx.x; c < nk; c += NT) kc[c] = (T)ys[nq + c];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int g = wave; g < a.G; g += NT / 64) {
-    const float* v = ys + nq + nk + g * a.dv;
-    float sq = 0.f;
-    for (int e = lane; e < a.dv; e += 64) sq += v[e] * v[e];
-    const float r = 1.f / sqrtf(wave_sum(sq) / (float)a.dv + a.v_eps);
-    for (int e = lane; e < a.dv; e += 64) vc[g * a.dv + e] = (T)(v[e] * r);
+  float r = 1.f;
+  if (vhead) r = 1.f / sqrtf(block_sum<CQ>(sq, scratch) / (float)a.dv + a.v_eps);     // (unit-uniform branch)
+  if (!dst_out) return;
+#pragma unroll
+  for (int u = 0; u < CQ_PER; ++u) {
+    const int e = threadIdx.x + u * CQ;
+    if (e < width) dst_out[e] = (T)(y[u] * r);
   }
 }
 
@@ -260,7 +284,8 @@ void launch_hyper_mix_norm(const HyperMixArgs& a, int f32, hipStream_t s) {
 
 void launch_conv_qkv_cache(const ConvQkvArgs& a, int f32, hipStream_t s) {
   if (a.T <= 0) return;
-  DISPATCH_T(f32, conv_qkv_cache_kernel<T><<<a.T, NT, (size_t)a.C * sizeof(float), s>>>(a);)
+  dim3 grid(a.T, a.H + 2 * a.G);
+  DISPATCH_T(f32, conv_qkv_cache_kernel<T><<<grid, CQ, 0, s>>>(a);)
 }
 
 void launch_memory_norm_gate(const float* y, const float* m, const void* gate, long long ldg, const float* w, float eps,
