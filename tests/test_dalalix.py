@@ -538,6 +538,35 @@ def test_convolved_projections_with_carried_taps(device, taps):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_convolved_projections_long_prompt(device):
+    """A prompt step of thousands of rows: two runs in one step, the second continuing its sequence from the slot."""
+    say("op conv_qkv_cache long", device)
+    torch.manual_seed(11)
+    H, G, dk, dv, BS, taps = 2, 2, 12, 20, 64, 4
+    C_ = H * dk + G * dk + G * dv
+    na, nb_ = 1500, 700
+    za, zb, w = torch.randn(na, C_), torch.randn(nb_ + 3, C_), torch.randn(C_, taps) * 0.7
+    ya, yb = O.short_conv(za.double(), w.double()), O.short_conv(zb.double(), w.double())[3:]
+    state = torch.full((3, taps - 1, C_), 1e4)
+    state[0] = zb[:3]
+    NB, bt, pos, slots = _paged(na + nb_, BS, 4)
+    prev, save, rs, cu, runs = _two_runs(na, nb_, True, False)
+    kc, vc, q = torch.zeros(NB, BS, G, dk), torch.zeros(NB, BS, G, dv), torch.empty(na + nb_, H, dk)
+    z = torch.cat([za, zb[3:]])
+    z, wd, state, slots, q, kc, vc, prev, save, rs, cu = _dev(device, z, w, state, slots, q, kc, vc, prev, save, rs, cu)
+    ops.conv_qkv_cache(z, wd, state, cu, rs, prev, runs, H, G, dk, dv, 1e-5, slots, q, kc, vc)
+    ops.conv_state_update(z, state, cu, prev, save, runs)
+    y = torch.cat([ya, yb])
+    rows = slots.cpu().long()
+    assert float((q.cpu().double().reshape(na + nb_, -1) - y[:, :H * dk]).abs().max()) < 1e-4
+    assert float((kc.cpu().view(-1, G * dk)[rows].double() - y[:, H * dk:(H + G) * dk]).abs().max()) < 1e-4
+    want_v = O.unit_rms(y[:, (H + G) * dk:].view(-1, G, dv), 1e-5).reshape(na + nb_, -1)
+    assert float((vc.cpu().view(-1, G * dv)[rows].double() - want_v).abs().max()) < 1e-4
+    assert float((state[0].cpu().double() - zb[-3:].double()).abs().max()) == 0.0
+    assert float((state[2].cpu().double() - za[-3:].double()).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_half_layout_rotation_and_cache_write(device):
     """Bias, rotation of the first dims entries of each head (entry i with i + dims / 2), the rest passing; no rotation
     and no bias where none is given."""
