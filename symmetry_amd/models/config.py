@@ -817,9 +817,10 @@ class DalalixConfig:
         return any(layer.mlp is not None for layer in self.layers)
 
     def owner(self, i: int) -> int:
-        """The layer whose tensors layer i reads."""
-        w = self.layers[i].weights_of
-        return i if w is None else w
+        """The layer whose tensors layer i reads (a borrowed layer may itself borrow: the chain ends at an owner)."""
+        while self.layers[i].weights_of is not None:
+            i = self.layers[i].weights_of
+        return i
 
     def attn_spec(self, i: int):
         """The softmax-attention part of layer i's mixer (every layer has one)."""
@@ -901,9 +902,8 @@ def dalalix_from_config(cfg: dict, name: str = "dalalix") -> DalalixConfig:
         layer = DalalixLayer(kind, mix, ff, None if wof is None else int(wof))
         if layer.weights_of is not None:
             src = layers[layer.weights_of] if 0 <= layer.weights_of < i else None
-            if src is None or src.weights_of is not None or (src.type, src.mixer, src.mlp) != (kind, mix, ff):
-                raise ValueError(f"layer {i}: weights_of {wof} must name an earlier layer of the same sizes with tensors "
-                                 "of its own")
+            if src is None or (src.type, src.mixer, src.mlp) != (kind, mix, ff):
+                raise ValueError(f"layer {i}: weights_of {wof} must name an earlier layer of the same kind and sizes")
         layers.append(layer)
     vocab, width, norm, _, _, emb, streams, cap, bos, eos = _take(
         cfg, "config", "vocab", "width", "norm", "layers",

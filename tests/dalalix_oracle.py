@@ -237,7 +237,10 @@ def forward(W, cfg, tokens, layers_out=None, margins=None):
     S = cfg.get("streams")
     X = [e.clone() for _ in range(S or 1)]
     for i, L in enumerate(cfg["layers"]):
-        p = f"l{L['weights_of']}." if L.get("weights_of") is not None else f"l{i}."
+        j = i
+        while cfg["layers"][j].get("weights_of") is not None:      # (a borrowed layer may itself borrow)
+            j = cfg["layers"][j]["weights_of"]
+        p = f"l{j}."
         subs = [(1, lambda h: mixer(W, cfg, L, p, h, positions))]
         if L.get("mlp") is not None:
             subs.append((2, lambda h: moe(W, p + "mlp.", L["mlp"], h, margins)))

@@ -54,7 +54,7 @@ def moe(experts=6, top=2, ff=12, limit=1.5, groups=3, keep=2):
 
 def cfg_mixed(width=40, vocab=67):
     """Every branch once: three streams, the pair table, all three mixers, a layer without feed-forward, layers that
-    borrow weights (a windowed one and a convolving one, so cache, memory and taps are the borrower's own), windows
+    borrow weights (windowed ones and a convolving one, so cache, memory and taps are the borrower's own), windows
     shorter and longer than the prompts, rotation on part of the head; all head sizes different from one another."""
     m1, m2, f1 = pair(), convd(), moe()
     layers = (
@@ -65,6 +65,7 @@ def cfg_mixed(width=40, vocab=67):
         C.DalalixLayer("parallel", pair(heads=2, kv=1, dim=8, vdim=16, window=200, keep=0, dims=8, mh=1, mn=20, mp=3, cap=3.0),
                        moe(experts=5, top=3, ff=8, groups=1, keep=1)),
         C.DalalixLayer("attention", m2, None, weights_of=2),
+        C.DalalixLayer("parallel", m1, f1, weights_of=3),          # borrows from a borrower: layer 1's tensors
     )
     return C.DalalixConfig(name="t-mixed", vocab_size=vocab, hidden_size=width, layers=layers, streams=3,
                            bigram=C.HashPairSpec(29, 7, 3), logit_softcap=4.0, norm_eps=1e-5)
@@ -114,11 +115,11 @@ def checkpoint(cfg, tmp_path, seed=0, sharpen=None):
     return path, C.dalalix_to_config(cfg), {k: v.to(torch.bfloat16) for k, v in w.tensors.items()}
 
 
-def engine(path, device, dtype, blocks=24, seqs=4, block_size=16, graphs=True):
+def engine(path, device, dtype, blocks=24, seqs=4, block_size=16, graphs=True, pipeline=False):
     return LLMEngine(EngineConfig(model="t", weights=path, dtype=dtype, device=device, max_num_seqs=seqs,
                                   block_size=block_size, num_kv_blocks=blocks + 1, max_model_len=blocks * block_size,
                                   max_num_batched_tokens=8192, use_graphs=graphs, enable_prefix_caching=False,
-                                  pipeline=False))
+                                  pipeline=pipeline))
 
 
 def tokens(n, vocab, seed):
@@ -337,6 +338,27 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device):
         for j, t in enumerate(out):
             top = lg[j].topk(2).values
             assert float(lg[j].max() - lg[j][t]) <= 1e-3 * float(lg[j].std()) or float(top[0] - top[1]) < 1e-3, (i, j)
+
+
+@pytest.mark.gpu
+def test_pipelined_decode_takes_the_previous_token_from_the_device(tmp_path):
+    """Pipelined decode: a step's input token is the sample the step before left on the device, and so is the token
+    the pair table hashes it with; the outputs equal those of the engine that waits for every step."""
+    cfg = cfg_mixed()
+    path, cj, W = checkpoint(cfg, tmp_path, seed=12)
+    prompts = [tokens(n, cfg.vocab_size, 40 + i) for i, n in enumerate((7, 21, 3))]
+    outs = {}
+    for pipe in (False, True):
+        eng = engine(path, "cuda", "float32", blocks=12, seqs=3, pipeline=pipe)
+        for i, p in enumerate(prompts):
+            eng.add_request(f"r{i}", p, SamplingParams(max_tokens=20, ignore_eos=True))
+        res = {}
+        while eng.has_unfinished():
+            for o in eng.step():
+                if o.finished:
+                    res[o.request_id] = list(o.seq.output_ids)
+        outs[pipe] = res
+    assert outs[True] == outs[False] and all(len(v) == 20 for v in outs[True].values())
 
 
 def test_config_reader_rejects_unknown_keys_and_roundtrips(tmp_path):
